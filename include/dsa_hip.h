@@ -1,0 +1,138 @@
+/*
+ * C ABI of the MI355X (gfx950) fused DeepSeek-Sparse-Attention kernels.
+ *
+ * One entry point per external kernel the reference's DSA path calls.  Every function takes raw
+ * device pointers plus sizes and a HIP stream (passed as void*; NULL = the null stream), launches
+ * asynchronously on that stream, allocates nothing, keeps no state between calls and returns an
+ * int status: 0 on success, negative on error (see dsa_last_error()).  All tensors are dense and
+ * row-major ("contiguous") unless a leading dimension is given.  Paths in the comments are
+ * relative to the reference tree.
+ */
+#ifndef DSA_HIP_H
+#define DSA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DSA_OK 0
+#define DSA_ERR_BAD_ARG (-1)     /* shape / alignment / unsupported size */
+#define DSA_ERR_LAUNCH (-2)      /* HIP reported a launch error */
+#define DSA_ERR_WORKSPACE (-3)   /* caller-provided workspace too small */
+
+/* ABI version; bumped whenever a signature changes. */
+int dsa_version(void);
+/* Human-readable description of the last error on the calling thread ("" if none). */
+const char* dsa_last_error(void);
+
+/*
+ * Row-wise e4m3 quantiser: amax -> max(amax, eps) -> scale = 448/amax (floored to a power of two
+ * when pow2 != 0) -> x8 = e4m3_rne(clamp(x * scale)), scale_inv = 1/scale.
+ * Replaces TransformerEngine's Float8BlockQuantizer as configured at
+ * loongforge/models/common/experimental_attention_variant/dsa_fused_kernels.py:2308-2315 and
+ * used at :2341-2346 (1x128 blocks => one scale per row of `cols` = 128 elements).
+ *   x        [rows, cols] bf16     x8 [rows, cols] fp8-e4m3 (OCP)     scale_inv [rows] f32
+ */
+int dsa_quant_rowwise_e4m3(const void* x, int64_t rows, int cols, void* x8, float* scale_inv,
+                           float eps, int pow2, void* stream);
+
+/*
+ * Lightning-indexer logits:
+ *   logits[i, j - base_i] = k_scale[j] * sum_h q_w[i,h] * relu(q8[i,h,:] . k8[j,:]),  ks[i] <= j < ke[i]
+ * and -inf for every other column of row i.  base_i = 0 when `relative` == 0 (dense layout, width
+ * Sk) and ks[i] when `relative` != 0 (packed layout of the reference, width = max_seqlen_k).
+ * Replaces deep_gemm.fp8_mqa_logits as called at dsa_fused_kernels.py:2366 and :2370-2380.
+ *   q8 [S, Hi, 128] e4m3   q_w [S, Hi] f32 (= weights * q_scale * 128^-0.5)   k8 [Sk, 128] e4m3
+ *   k_scale [Sk] f32   ks, ke [S] i32   logits [S, ld] f32 (ld >= width)
+ */
+int dsa_indexer_logits(const void* q8, const float* q_w, const void* k8, const float* k_scale,
+                       const int32_t* ks, const int32_t* ke, int S, int Hi, int Sk,
+                       float* logits, int64_t ld, int width, int relative, void* stream);
+
+/*
+ * Per-row top-k by value.  Row i considers columns [0, row_len[i]) of logits (row_len == NULL:
+ * `width` for every row); -inf entries are never selected.  Outputs K slots per row: the selected
+ * scores (descending when `sorted` != 0, otherwise in ascending column order) and column ids +
+ * id_base[i] (id_base == NULL: 0); unused slots hold score -inf and id -1.
+ * Replaces flashinfer.top_k behind padded_flashinfer_topk, dsa_fused_kernels.py:1958-1998, and the
+ * id globalisation at :2386-2387.
+ *   logits [S, ld] f32   scores [S, K] f32   ids [S, K] i32
+ */
+int dsa_topk(const float* logits, int S, int width, int64_t ld, const int32_t* row_len,
+             const int32_t* id_base, int K, int sorted, float* scores, int32_t* ids, void* stream);
+
+/*
+ * Fused indexer forward = dsa_indexer_logits + dsa_topk without a caller-visible [S, Sk] matrix:
+ * `workspace` (>= dsa_indexer_topk_workspace_bytes) holds the logits of one query block at a time.
+ * Replaces DSAIndexerKernelFunction.forward after quantisation, dsa_fused_kernels.py:2348-2387.
+ * ids are global key rows; rows with fewer than K visible keys are padded with id -1 / score -inf.
+ */
+size_t dsa_indexer_topk_workspace_bytes(int S, int Sk, int K);
+int dsa_indexer_topk_fwd(const void* q8, const float* q_w, const void* k8, const float* k_scale,
+                         const int32_t* ks, const int32_t* ke, int S, int Hi, int Sk, int K,
+                         int sorted, float* scores, int32_t* ids, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
+/*
+ * Sparse gradients of the selected logits w.r.t. the fp8 payloads and the scaled weights
+ * (scales are constants):  with j = ids[i,t] >= 0, r_h = q8[i,h,:] . k8[j,:],
+ *   d_qw[i,h]   = sum_t g[i,t] k_scale[j] relu(r_h)
+ *   d_q8[i,h,:] = sum_t g[i,t] k_scale[j] q_w[i,h] [r_h > 0] k8[j,:]
+ *   d_k8[j,:]   = sum_{(i,t): ids[i,t]=j} g[i,t] k_scale[j] sum_h q_w[i,h] [r_h > 0] q8[i,h,:]
+ * d_k8 is accumulated in a fixed order (bit-reproducible).  Replaces
+ * lightning_indexer_bwd.fp8_mqa_logits_bwd as called at dsa_fused_kernels.py:2421-2430.
+ *   g [S, K] f32   d_q8 [S, Hi, 128] f32   d_k8 [Sk, 128] f32   d_qw [S, Hi] f32
+ */
+size_t dsa_indexer_bwd_workspace_bytes(int S, int Hi, int Sk, int K);
+int dsa_indexer_bwd(const float* g, const void* q8, const void* k8, const float* k_scale,
+                    const float* q_w, const int32_t* ids, int S, int Hi, int Sk, int K,
+                    float* d_q8, float* d_k8, float* d_qw, void* workspace, size_t workspace_bytes,
+                    void* stream);
+
+/*
+ * Sparse MQA-MLA attention forward.  Slot t of query i (global position q_start + i) is valid iff
+ * ids[i,t] != -1, 0 <= ids[i,t] < Skv and ids[i,t] <= q_start + i.  Over the valid slots:
+ *   s = q[i,h,:] . kv[ids[i,t],:]   P = softmax_t(s * sm_scale)   out[i,h,:] = sum_t P kv[ids[i,t], :d_v]
+ *   lse[i,h] = natural-log sum-exp of s * sm_scale  (+inf, with out = 0, when no slot is valid)
+ *   p_out[i,h,t] = s (raw logit) on valid slots, -inf elsewhere; optional (NULL to skip);
+ *                  p_out_f32 selects f32 (1) or bf16 (0) storage.
+ * Replaces flash_mla_fwd.flash_mla_sparse_fwd as called at dsa_fused_kernels.py:2048-2059
+ * (math: ops/tilelang_ops/sparse_mla_fwd.py:129-180).
+ *   q [S, H, 576] bf16   kv [Skv, 576] bf16   ids [S, K] i32 (K % 64 == 0)
+ *   out [S, H, 512] bf16   lse [S, H] f32   p_out [S, H, K]
+ */
+int dsa_sparse_mla_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv,
+                       int K, int q_start, float sm_scale, int d_v, void* out, float* lse,
+                       void* p_out, int p_out_f32, void* stream);
+
+/*
+ * Sparse MQA-MLA attention backward: dQ and dKV of dsa_sparse_mla_fwd given dO, the saved out and
+ * natural-log lse.  dKV is accumulated in fp32 in a fixed order (bit-reproducible, no float
+ * atomics) and returned as bf16.  Replaces flash_mla_bwd.flash_mla_sparse_bwd /
+ * sparse_mla_bwd_interface as called at dsa_fused_kernels.py:2086-2110
+ * (math: loongforge/models/common/experimental_attention_variant/sparse_mla_bwd.py:292-356).
+ *   dout [S, H, 512] bf16   dq [S, H, 576] bf16   dkv [Skv, 576] bf16
+ */
+size_t dsa_sparse_mla_bwd_workspace_bytes(int S, int H, int Skv, int K);
+int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out, const void* dout,
+                       const int32_t* ids, const float* lse, int S, int H, int Skv, int K,
+                       int q_start, float sm_scale, int d_v, void* dq, void* dkv,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Head-averaged attention distribution over the selected slots:
+ *   target[i,t] = (1/H) sum_h softmax_t(p_out[i,h,:] * sm_scale)[t]
+ * Replaces triton_attn_dist, dsa_fused_kernels.py:1844-1955.  `ld_s` / `ld_h` are the element
+ * strides of p_out between queries / heads (so a head-sliced view can be passed).
+ *   p_out [S, H, K] bf16 or f32   target [S, K] f32
+ */
+int dsa_attn_dist(const void* p_out, int p_out_f32, int S, int H, int K, int64_t ld_s,
+                  int64_t ld_h, float sm_scale, float* target, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DSA_HIP_H */

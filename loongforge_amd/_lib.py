@@ -1,0 +1,65 @@
+"""ctypes binding of libdsa_hip.so, the C-ABI library of gfx950 kernels.
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+import ctypes
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdsa_hip.so")
+
+_c = ctypes
+_vp, _i, _i64, _f, _sz = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float, _c.c_size_t
+
+# name -> (restype, argtypes); mirrors include/dsa_hip.h
+SIGNATURES = {
+    "dsa_version": (_i, []),
+    "dsa_last_error": (_c.c_char_p, []),
+    "dsa_quant_rowwise_e4m3": (_i, [_vp, _i64, _i, _vp, _vp, _f, _i, _vp]),
+    "dsa_indexer_logits": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i64, _i, _i, _vp]),
+    "dsa_topk": (_i, [_vp, _i, _i, _i64, _vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "dsa_indexer_topk_workspace_bytes": (_sz, [_i, _i, _i]),
+    "dsa_indexer_topk_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _sz, _vp]),
+    "dsa_indexer_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "dsa_indexer_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "dsa_sparse_mla_fwd": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _i, _vp]),
+    "dsa_sparse_mla_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "dsa_sparse_mla_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _sz, _vp]),
+    "dsa_attn_dist": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _f, _vp, _vp]),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+class DsaError(RuntimeError):
+    """A kernel launch failed or the library rejected its arguments."""
+
+
+def load():
+    """Loads the shared library (once) and declares every entry point's signature."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise DsaError(
+                "libdsa_hip.so is missing at %s; build it with `python -m loongforge_amd.csrc.build` "
+                "(there is no fallback implementation)" % LIB_PATH)
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)      # AttributeError if a declared symbol is not exported
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+        return _lib
+
+
+def check(rc, what):
+    """Turns a negative status into an exception carrying dsa_last_error()."""
+    if rc != 0:
+        msg = load().dsa_last_error().decode("utf-8", "replace")
+        if rc == -1:
+            raise ValueError("%s: %s" % (what, msg))
+        raise DsaError("%s failed (status %d): %s" % (what, rc, msg))

@@ -1,0 +1,91 @@
+// Head-averaged softmax over the selected slots: target[i,t] = mean_h softmax_t(p_out[i,h,:] * c).
+// HBM-bound: reads H*K logits per query once.  One workgroup per query; each wave takes heads
+// w, w+4, ...; a head's K logits live in registers (K/64 per lane), so p_out is read exactly once.
+#include "dsa_common.h"
+
+namespace {
+
+constexpr int MAXV = 64;   // slots per lane: supports K <= 4096
+
+template <bool F32>
+__device__ __forceinline__ float load_logit(const void* p, int64_t off) {
+  if (F32) return ((const float*)p)[off];
+  return bf16_bits_to_f32(((const unsigned short*)p)[off]);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+template <bool F32, int NV>
+__global__ __launch_bounds__(256) void attn_dist_kernel(const void* __restrict__ p_out, int H, int K,
+                                                        int64_t ld_s, int64_t ld_h, float c2,
+                                                        float* __restrict__ target) {
+  extern __shared__ float acc_s[];            // [4 waves][K]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t i = blockIdx.x;
+  float acc[NV];
+#pragma unroll
+  for (int v = 0; v < NV; v++) acc[v] = 0.f;
+  for (int h = wave; h < H; h += 4) {
+    const int64_t base = i * ld_s + h * ld_h;
+    float z[NV];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+      int t = v * 64 + lane;
+      z[v] = t < K ? load_logit<F32>(p_out, base + t) * c2 : -INFINITY;
+      mx = fmaxf(mx, z[v]);
+    }
+    mx = wave_max(mx);
+    if (mx == -INFINITY) continue;            // head with no valid slot contributes nothing
+    float sum = 0.f;
+#pragma unroll
+    for (int v = 0; v < NV; v++) { z[v] = exp2f(z[v] - mx); sum += z[v]; }
+    sum = wave_sum(sum);
+    float inv = 1.0f / sum;
+#pragma unroll
+    for (int v = 0; v < NV; v++) acc[v] += z[v] * inv;
+  }
+#pragma unroll
+  for (int v = 0; v < NV; v++) { int t = v * 64 + lane; if (t < K) acc_s[wave * K + t] = acc[v]; }
+  __syncthreads();
+  const float invh = 1.0f / (float)H;
+  for (int t = threadIdx.x; t < K; t += 256)
+    target[i * K + t] = ((acc_s[t] + acc_s[K + t]) + (acc_s[2 * K + t] + acc_s[3 * K + t])) * invh;
+}
+
+template <bool F32>
+int launch(const void* p_out, int S, int H, int K, int64_t ld_s, int64_t ld_h, float sm_scale, float* target,
+           hipStream_t st) {
+  const float c2 = sm_scale * 1.4426950408889634f;
+  size_t smem = (size_t)4 * K * sizeof(float);
+  int nv = (K + 63) / 64;
+#define DSA_AD_CASE(N) \
+  if (nv <= N) { attn_dist_kernel<F32, N><<<dim3(S), dim3(256), smem, st>>>(p_out, H, K, ld_s, ld_h, c2, target); return 0; }
+  DSA_AD_CASE(1) DSA_AD_CASE(2) DSA_AD_CASE(4) DSA_AD_CASE(8) DSA_AD_CASE(16) DSA_AD_CASE(32) DSA_AD_CASE(64)
+#undef DSA_AD_CASE
+  return -1;
+}
+
+}  // namespace
+
+extern "C" int dsa_attn_dist(const void* p_out, int p_out_f32, int S, int H, int K, int64_t ld_s, int64_t ld_h,
+                             float sm_scale, float* target, void* stream) {
+  DSA_REQUIRE(S >= 0 && H > 0 && K > 0, "dsa_attn_dist: bad shape S=%d H=%d K=%d", S, H, K);
+  DSA_REQUIRE(K <= 64 * MAXV, "dsa_attn_dist: K=%d exceeds the supported maximum %d", K, 64 * MAXV);
+  DSA_REQUIRE(ld_h >= K && ld_s >= ld_h, "dsa_attn_dist: bad strides");
+  if (S == 0) return DSA_OK;
+  int rc = p_out_f32 ? launch<true>(p_out, S, H, K, ld_s, ld_h, sm_scale, target, (hipStream_t)stream)
+                     : launch<false>(p_out, S, H, K, ld_s, ld_h, sm_scale, target, (hipStream_t)stream);
+  DSA_REQUIRE(rc == 0, "dsa_attn_dist: unsupported K");
+  DSA_CHECK_LAUNCH("dsa_attn_dist");
+  return DSA_OK;
+}

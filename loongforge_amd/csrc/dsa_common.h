@@ -1,0 +1,45 @@
+// Shared device/host helpers for the gfx950 DSA kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/dsa_hip.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// ---- error plumbing (never throws across the C ABI) ------------------------------------
+void dsa_set_error(const char* fmt, ...);
+#define DSA_FAIL(code, ...) do { dsa_set_error(__VA_ARGS__); return (code); } while (0)
+#define DSA_REQUIRE(cond, ...) do { if (!(cond)) DSA_FAIL(DSA_ERR_BAD_ARG, __VA_ARGS__); } while (0)
+#define DSA_CHECK_LAUNCH(name) do { hipError_t e_ = hipGetLastError(); \
+    if (e_ != hipSuccess) DSA_FAIL(DSA_ERR_LAUNCH, "%s: launch failed: %s", name, hipGetErrorString(e_)); } while (0)
+
+// ---- small device helpers ----------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(unsigned short h) {
+  return __builtin_bit_cast(float, ((unsigned)h) << 16);
+}
+__device__ __forceinline__ unsigned short f32_to_bf16_bits(float f) {   // round-to-nearest-even
+  unsigned u = __builtin_bit_cast(unsigned, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (unsigned short)(u >> 16);
+}
+__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
+  return (unsigned)f32_to_bf16_bits(lo) | ((unsigned)f32_to_bf16_bits(hi) << 16);
+}
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding).
+#define DSA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 0xf) | (((n) >> 4) << 14)) | (0x7 << 4) | (0xf << 8))
+
+static inline int dsa_cdiv(long a, long b) { return (int)((a + b - 1) / b); }

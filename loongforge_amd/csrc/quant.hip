@@ -1,0 +1,66 @@
+// Row-wise e4m3 quantiser (one power-of-two scale per 128-element row).
+// HBM-bound: reads 2 B and writes 1 B per element plus 4 B per row; one 64-lane wave per row
+// group, each lane handling 8 consecutive elements (16-byte loads, 8-byte stores).
+#include "dsa_common.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_max16(float v) {   // max over the 16 lanes sharing a row
+  v = fmaxf(v, __shfl_xor(v, 1, 64));
+  v = fmaxf(v, __shfl_xor(v, 2, 64));
+  v = fmaxf(v, __shfl_xor(v, 4, 64));
+  v = fmaxf(v, __shfl_xor(v, 8, 64));
+  return v;
+}
+
+// cols == 128: 16 lanes per row, 4 rows per wave, 16 rows per 256-thread block.
+__global__ __launch_bounds__(256) void quant128_kernel(const uint4* __restrict__ x, uint2* __restrict__ x8,
+                                                       float* __restrict__ scale_inv, int64_t rows,
+                                                       float eps, int pow2) {
+  int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  int sub = threadIdx.x & 15;
+  bool live = row < rows;
+  uint4 raw = live ? x[row * 16 + sub] : make_uint4(0, 0, 0, 0);
+  unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+    v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(v[i]));
+  amax = wave_max16(amax);
+  amax = fmaxf(amax, eps);
+  float scale = 448.0f / amax;                       // correctly rounded fp32 division
+  if (pow2) scale = __builtin_bit_cast(float, __builtin_bit_cast(unsigned, scale) & 0xff800000u);
+  float q[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) q[i] = fminf(fmaxf(v[i] * scale, -448.0f), 448.0f);  // cvt does not saturate
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], hi, true);
+  if (live) {
+    x8[row * 16 + sub] = make_uint2((unsigned)lo, (unsigned)hi);
+    if (sub == 0) scale_inv[row] = 1.0f / scale;
+  }
+}
+
+}  // namespace
+
+extern "C" int dsa_quant_rowwise_e4m3(const void* x, int64_t rows, int cols, void* x8, float* scale_inv,
+                                      float eps, int pow2, void* stream) {
+  DSA_REQUIRE(cols == 128, "dsa_quant_rowwise_e4m3: only rows of 128 elements are supported, got %d", cols);
+  DSA_REQUIRE(rows >= 0, "dsa_quant_rowwise_e4m3: negative row count");
+  DSA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)x8 % 8) == 0, "dsa_quant_rowwise_e4m3: misaligned pointer");
+  if (rows == 0) return DSA_OK;
+  int64_t blocks = (rows + 15) / 16;
+  DSA_REQUIRE(blocks < (1ll << 31), "dsa_quant_rowwise_e4m3: too many rows");
+  quant128_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+      (const uint4*)x, (uint2*)x8, scale_inv, rows, eps, pow2);
+  DSA_CHECK_LAUNCH("dsa_quant_rowwise_e4m3");
+  return DSA_OK;
+}
