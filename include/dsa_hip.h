@@ -53,16 +53,18 @@ int dsa_indexer_logits(const void* q8, const float* q_w, const void* k8, const f
                        float* logits, int64_t ld, int width, int relative, void* stream);
 
 /*
- * Per-row top-k by value.  Row i considers columns [0, row_len[i]) of logits (row_len == NULL:
- * `width` for every row); -inf entries are never selected.  Outputs K slots per row: the selected
- * scores (descending when `sorted` != 0, otherwise in ascending column order) and column ids +
- * id_base[i] (id_base == NULL: 0); unused slots hold score -inf and id -1.
+ * Per-row top-k by value.  Row i considers columns [row_begin[i], row_end[i]) of logits, clipped to
+ * [0, width) (NULL: 0 / width for every row); -inf entries are never selected.  Outputs K slots per
+ * row: the selected scores (descending when `sorted` != 0, otherwise in ascending column order) and
+ * column ids + id_base[i] (id_base == NULL: 0); unused slots hold score -inf and id -1.  Ties at the
+ * K-th value are broken towards the lower column, so the result is deterministic.
  * Replaces flashinfer.top_k behind padded_flashinfer_topk, dsa_fused_kernels.py:1958-1998, and the
  * id globalisation at :2386-2387.
  *   logits [S, ld] f32   scores [S, K] f32   ids [S, K] i32
  */
-int dsa_topk(const float* logits, int S, int width, int64_t ld, const int32_t* row_len,
-             const int32_t* id_base, int K, int sorted, float* scores, int32_t* ids, void* stream);
+int dsa_topk(const float* logits, int S, int64_t ld, const int32_t* row_begin, const int32_t* row_end,
+             int width, const int32_t* id_base, int K, int sorted, float* scores, int32_t* ids,
+             void* stream);
 
 /*
  * Fused indexer forward = dsa_indexer_logits + dsa_topk without a caller-visible [S, Sk] matrix:

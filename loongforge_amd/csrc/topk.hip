@@ -1,0 +1,247 @@
+// Per-row top-k selection (radix select with the candidate histograms in LDS) for gfx950.
+//
+// One workgroup per row.  The row's window is read from HBM exactly once into LDS as
+// order-preserving 32-bit keys; three histogram passes (12 + 10 + 10 bits, most significant first)
+// locate the k-th largest key exactly, a prefix-sum compaction then emits every key above it plus
+// the first ties in ascending column order, so the result is deterministic.  An optional bitonic
+// sort in LDS orders the K outputs by descending score.  HBM-bound by design: 4 bytes read per
+// candidate, 8 bytes written per output slot; everything else stays in LDS.
+#include "dsa_common.h"
+
+namespace {
+
+constexpr int BLOCK = 256;
+constexpr int NW = BLOCK / 64;
+constexpr int HBINS = 4096;
+
+__device__ __forceinline__ unsigned f2key(float f) {       // larger float <-> larger unsigned
+  unsigned u = __builtin_bit_cast(unsigned, f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key2f(unsigned k) {
+  unsigned u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __builtin_bit_cast(float, u);
+}
+
+// exclusive prefix sum over the block (thread order), also returns the block total
+__device__ __forceinline__ int block_exscan(int v, int* scratch, int& total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int inc = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    int n = __shfl_up(inc, o, 64);
+    if (lane >= o) inc += n;
+  }
+  __syncthreads();
+  if (lane == 63) scratch[wave] = inc;
+  __syncthreads();
+  int base = 0, tot = 0;
+#pragma unroll
+  for (int w = 0; w < NW; w++) { int s = scratch[w]; if (w < wave) base += s; tot += s; }
+  total = tot;
+  return base + inc - v;
+}
+
+struct Pick { int bin; int above; };
+
+// Finds, scanning bins from the highest down, the bin in which the running count reaches `need`.
+// hist has nb bins (nb % BLOCK == 0).  Result: that bin and the number of keys in higher bins.
+__device__ __forceinline__ Pick pick_bin(const int* hist, int nb, int need, int* scratch, int* res) {
+  const int per = nb / BLOCK;
+  const int hi = nb - 1 - (int)threadIdx.x * per;          // this thread owns bins hi, hi-1, ..., hi-per+1
+  int local = 0;
+  for (int b = 0; b < per; b++) local += hist[hi - b];
+  int total;
+  int before = block_exscan(local, scratch, total);
+  if (before < need && before + local >= need) {
+    int run = before;
+    for (int b = 0; b < per; b++) {
+      int c = hist[hi - b];
+      if (run + c >= need) { res[0] = hi - b; res[1] = run; break; }
+      run += c;
+    }
+  }
+  __syncthreads();
+  Pick p = {res[0], res[1]};
+  __syncthreads();
+  return p;
+}
+
+template <bool STAGED>
+__global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ logits, long ld,
+                                                     const int* __restrict__ row_begin, const int* __restrict__ row_end,
+                                                     int width, const int* __restrict__ id_base, int K, int Kp2, int sorted,
+                                                     float* __restrict__ scores, int* __restrict__ ids, int nmax) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  int* hist = (int*)smem;                          // HBINS
+  int* scratch = hist + HBINS;                     // 16
+  float* outv = (float*)(scratch + 16);            // Kp2
+  int* outi = (int*)(outv + Kp2);                  // Kp2
+  unsigned* keys = (unsigned*)(outi + Kp2);        // nmax (STAGED only)
+  const int tid = threadIdx.x;
+  const long row = blockIdx.x;
+  const int cb = max(row_begin ? row_begin[row] : 0, 0);
+  const int ce = min(row_end ? row_end[row] : width, width);
+  const int n = max(ce - cb, 0);
+  const int base_id = (id_base ? id_base[row] : 0) + cb;
+  const float* src = logits + row * ld + cb;
+  float* sv = scores + row * (long)K;
+  int* si = ids + row * (long)K;
+  (void)nmax;
+
+  auto key_at = [&](int e) -> unsigned { return STAGED ? keys[e] : f2key(src[e]); };
+
+  if (n <= K) {
+    for (int t = tid; t < Kp2; t += BLOCK) {
+      float v = t < n ? src[t] : -INFINITY;
+      outv[t] = v;
+      outi[t] = (t < n && v > -INFINITY) ? base_id + t : -1;
+    }
+  } else {
+    if (STAGED) {
+      for (int e = tid; e < n; e += BLOCK) keys[e] = f2key(src[e]);
+    }
+    // ---- pass 1: bits [31:20] ------------------------------------------------------------
+    for (int b = tid; b < HBINS; b += BLOCK) hist[b] = 0;
+    __syncthreads();
+    for (int e = tid; e < n; e += BLOCK) atomicAdd(&hist[key_at(e) >> 20], 1);
+    __syncthreads();
+    Pick p1 = pick_bin(hist, 4096, K, scratch, scratch + 8);
+    int need = K - p1.above;
+    // ---- pass 2: bits [19:10] among keys in bin p1 -----------------------------------------
+    for (int b = tid; b < 1024; b += BLOCK) hist[b] = 0;
+    __syncthreads();
+    for (int e = tid; e < n; e += BLOCK) {
+      unsigned k = key_at(e);
+      if ((int)(k >> 20) == p1.bin) atomicAdd(&hist[(k >> 10) & 1023], 1);
+    }
+    __syncthreads();
+    Pick p2 = pick_bin(hist, 1024, need, scratch, scratch + 8);
+    need -= p2.above;
+    // ---- pass 3: bits [9:0] ----------------------------------------------------------------
+    const unsigned pre22 = ((unsigned)p1.bin << 10) | (unsigned)p2.bin;
+    for (int b = tid; b < 1024; b += BLOCK) hist[b] = 0;
+    __syncthreads();
+    for (int e = tid; e < n; e += BLOCK) {
+      unsigned k = key_at(e);
+      if ((k >> 10) == pre22) atomicAdd(&hist[k & 1023], 1);
+    }
+    __syncthreads();
+    Pick p3 = pick_bin(hist, 1024, need, scratch, scratch + 8);
+    const unsigned thr = (pre22 << 10) | (unsigned)p3.bin;   // the K-th largest key
+    const int ties = need - p3.above;                         // how many keys == thr to keep (>= 1)
+    // ---- compaction in ascending column order ------------------------------------------------
+    const int cs = (n + BLOCK - 1) / BLOCK;
+    const int e0 = min(tid * cs, n), e1 = min(e0 + cs, n);
+    int ngt = 0, neq = 0;
+    for (int e = e0; e < e1; e++) { unsigned k = key_at(e); ngt += k > thr; neq += k == thr; }
+    int tot;
+    const int eq_before = block_exscan(neq, scratch, tot);
+    const int eq_take = max(0, min(neq, ties - eq_before));
+    int pos = block_exscan(ngt + eq_take, scratch, tot);
+    int eq_seen = 0;
+    for (int e = e0; e < e1; e++) {
+      unsigned k = key_at(e);
+      bool take = k > thr;
+      if (k == thr) { take = eq_seen < eq_take; eq_seen++; }
+      if (take) {
+        float v = key2f(k);
+        outv[pos] = v;
+        outi[pos] = v > -INFINITY ? base_id + e : -1;
+        pos++;
+      }
+    }
+    for (int t = K + tid; t < Kp2; t += BLOCK) { outv[t] = -INFINITY; outi[t] = -1; }
+  }
+  __syncthreads();
+
+  if (sorted) {   // bitonic sort, descending score, ascending id among equal scores
+    for (int size = 2; size <= Kp2; size <<= 1) {
+      for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        for (int t = tid; t < (Kp2 >> 1); t += BLOCK) {
+          const int lo = 2 * t - (t & (stride - 1));
+          const int hi = lo + stride;
+          const bool desc = ((lo & size) == 0);
+          const float a = outv[lo], b = outv[hi];
+          const int ia = outi[lo], ib = outi[hi];
+          const bool a_first = (a > b) || (a == b && (unsigned)ia < (unsigned)ib);   // id -1 sorts last
+          if (a_first != desc) { outv[lo] = b; outv[hi] = a; outi[lo] = ib; outi[hi] = ia; }
+        }
+        __syncthreads();
+      }
+    }
+  }
+  for (int t = tid; t < K; t += BLOCK) { sv[t] = outv[t]; si[t] = outi[t]; }
+}
+
+}  // namespace
+
+int dsa_topk_launch(const float* logits, int S, int64_t ld, const int32_t* row_begin, const int32_t* row_end,
+                    int width, const int32_t* id_base, int K, int sorted, float* scores, int32_t* ids,
+                    hipStream_t st) {
+  DSA_REQUIRE(S >= 0 && width > 0 && ld >= width && K > 0, "dsa_topk: bad sizes S=%d width=%d K=%d", S, width, K);
+  DSA_REQUIRE(K <= 8192, "dsa_topk: K=%d exceeds the supported maximum 8192", K);
+  if (S == 0) return DSA_OK;
+  int Kp2 = 1;
+  while (Kp2 < K) Kp2 <<= 1;
+  const size_t fixed = (size_t)HBINS * 4 + 64 + (size_t)Kp2 * 8;
+  const size_t staged = fixed + (size_t)width * 4;
+  const bool use_staged = staged <= 160 * 1024;
+  const size_t smem = use_staged ? staged : fixed;
+  auto kern = use_staged ? topk_kernel<true> : topk_kernel<false>;
+  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+    DSA_FAIL(DSA_ERR_LAUNCH, "dsa_topk: cannot reserve %zu bytes of LDS", smem);
+  kern<<<dim3(S), dim3(BLOCK), smem, st>>>(logits, (long)ld, row_begin, row_end, width, id_base, K, Kp2, sorted,
+                                           scores, ids, width);
+  DSA_CHECK_LAUNCH("dsa_topk");
+  return DSA_OK;
+}
+
+extern "C" int dsa_topk(const float* logits, int S, int64_t ld, const int32_t* row_begin, const int32_t* row_end,
+                        int width, const int32_t* id_base, int K, int sorted, float* scores, int32_t* ids,
+                        void* stream) {
+  return dsa_topk_launch(logits, S, ld, row_begin, row_end, width, id_base, K, sorted, scores, ids,
+                         (hipStream_t)stream);
+}
+
+// ---- fused indexer forward: logits of one query block at a time, then its top-k ----------------
+int dsa_indexer_logits_block(const void* q8, const float* q_w, const void* k8, const float* k_scale,
+                             const int32_t* ks, const int32_t* ke, int S, int Hi, int Sk, float* logits,
+                             int64_t ld, int width, int relative, int clean, int q_begin, int q_count,
+                             hipStream_t st);
+
+static int fused_block_rows(int Sk) {
+  // one block's logits stay within the 256 MiB memory-side cache, and a block still has enough
+  // workgroups (8 queries each) to cover all 256 compute units several times over
+  long rows = (256l << 20) / ((long)Sk * 4);
+  rows = rows < 2048 ? 2048 : rows;
+  return (int)(rows / 8 * 8);
+}
+
+extern "C" size_t dsa_indexer_topk_workspace_bytes(int S, int Sk, int K) {
+  (void)K;
+  int rows = fused_block_rows(Sk);
+  if (rows > S) rows = (S + 7) / 8 * 8;
+  return (size_t)rows * (size_t)Sk * 4;
+}
+
+extern "C" int dsa_indexer_topk_fwd(const void* q8, const float* q_w, const void* k8, const float* k_scale,
+                                    const int32_t* ks, const int32_t* ke, int S, int Hi, int Sk, int K, int sorted,
+                                    float* scores, int32_t* ids, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  if (S == 0) return DSA_OK;
+  DSA_REQUIRE(workspace != nullptr && workspace_bytes >= dsa_indexer_topk_workspace_bytes(S, Sk, K),
+              "dsa_indexer_topk_fwd: workspace of %zu bytes is too small", workspace_bytes);
+  int rows = fused_block_rows(Sk);
+  float* lg = (float*)workspace;
+  for (int q0 = 0; q0 < S; q0 += rows) {
+    const int cnt = S - q0 < rows ? S - q0 : rows;
+    int rc = dsa_indexer_logits_block(q8, q_w, k8, k_scale, ks, ke, S, Hi, Sk, lg, Sk, Sk, 0, 0, q0, cnt, st);
+    if (rc != DSA_OK) return rc;
+    rc = dsa_topk_launch(lg, cnt, Sk, ks + q0, ke + q0, Sk, nullptr, K, sorted, scores + (size_t)q0 * K,
+                         ids + (size_t)q0 * K, st);
+    if (rc != DSA_OK) return rc;
+  }
+  return DSA_OK;
+}
