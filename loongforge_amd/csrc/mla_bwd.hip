@@ -17,6 +17,7 @@
 // an exclusive scan over keys: integer work only, so the order - and with it every fp32 sum - is
 // identical from run to run.  No floating-point atomics anywhere.
 #include "mla_tile.h"
+#include "order.h"
 
 namespace {
 using namespace mla;
@@ -54,85 +55,6 @@ __device__ __forceinline__ void wait_vmcnt_le(int n) {
     C(38) C(39) C(40) C(41) C(42) C(43) C(44) C(45) C(46) C(47) C(48)
 #undef C
     default: DSA_WAIT_VMCNT(0); break;
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// pass 0: key-sorted order of the valid (query, slot) pairs
-// ---------------------------------------------------------------------------------------------
-__global__ void zero_u32_kernel(unsigned* __restrict__ p, size_t n) {
-  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) p[e] = 0u;
-}
-
-// bitmap[key][w] bit b  <=>  local query 32w + b selects key
-__global__ void bm_set_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv, int q_start,
-                              unsigned* __restrict__ bitmap, int W) {
-  const size_t n = (size_t)cnt * K;
-  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
-    const int ql = (int)(e / K);
-    const int v = ids[(size_t)(q0 + ql) * K + (e % K)];
-    if (v >= 0 && v < Skv && v <= q_start + q0 + ql) atomicOr(&bitmap[(size_t)v * W + (ql >> 5)], 1u << (ql & 31));
-  }
-}
-
-// prefix[key][w] = number of set bits in words < w; count[key] = total.  One wave per key.
-__global__ __launch_bounds__(256) void bm_prefix_kernel(const unsigned* __restrict__ bitmap, unsigned* __restrict__ prefix,
-                                                        int* __restrict__ count, int Skv, int W) {
-  const int lane = threadIdx.x & 63;
-  const int key = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (key >= Skv) return;
-  int run = 0;
-  for (int w0 = 0; w0 < W; w0 += 64) {
-    const int w = w0 + lane;
-    const int c = w < W ? __popc(bitmap[(size_t)key * W + w]) : 0;
-    int inc = c;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) { int n = __shfl_up(inc, o, 64); if (lane >= o) inc += n; }
-    if (w < W) prefix[(size_t)key * W + w] = (unsigned)(run + inc - c);
-    run += __shfl(inc, 63, 64);
-  }
-  if (lane == 0) count[key] = run;
-}
-
-// start[key] = exclusive prefix sum of count (single workgroup; Skv is at most a few 10^5)
-__global__ __launch_bounds__(1024) void key_scan_kernel(const int* __restrict__ count, int* __restrict__ start, int Skv) {
-  __shared__ int wsum[16];
-  __shared__ int carry_s;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid == 0) carry_s = 0;
-  __syncthreads();
-  for (int base = 0; base < Skv; base += 1024) {
-    const int k = base + tid;
-    const int c = k < Skv ? count[k] : 0;
-    int inc = c;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) { int n = __shfl_up(inc, o, 64); if (lane >= o) inc += n; }
-    if (lane == 63) wsum[wave] = inc;
-    __syncthreads();
-    int before = carry_s;
-    for (int w = 0; w < wave; w++) before += wsum[w];
-    if (k < Skv) start[k] = before + inc - c;
-    __syncthreads();
-    if (tid == 1023) carry_s = before + inc;
-    __syncthreads();
-  }
-  if (tid == 0) start[Skv] = carry_s;
-}
-
-// dst[ql][slot] = row of the pair in key-sorted order (-1 for invalid slots)
-__global__ void rank_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv, int q_start,
-                            const unsigned* __restrict__ bitmap, const unsigned* __restrict__ prefix,
-                            const int* __restrict__ start, int W, int* __restrict__ dst) {
-  const size_t n = (size_t)cnt * K;
-  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
-    const int ql = (int)(e / K);
-    const int v = ids[(size_t)(q0 + ql) * K + (e % K)];
-    int d = -1;
-    if (v >= 0 && v < Skv && v <= q_start + q0 + ql) {
-      const size_t wi = (size_t)v * W + (ql >> 5);
-      d = start[v] + (int)prefix[wi] + __popc(bitmap[wi] & ((1u << (ql & 31)) - 1u));
-    }
-    dst[e] = d;
   }
 }
 
@@ -684,12 +606,7 @@ extern "C" int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out
   bool first = true;
   for (int q0 = 0; q0 < S; q0 += p.chunk) {
     const int cnt = S - q0 < p.chunk ? S - q0 : p.chunk;
-    const size_t bm_words = (size_t)Skv * p.W;
-    zero_u32_kernel<<<dim3(1024), dim3(256), 0, st>>>(bitmap, bm_words);
-    bm_set_kernel<<<dim3(2048), dim3(256), 0, st>>>(ids, q0, cnt, K, Skv, q_start, bitmap, p.W);
-    bm_prefix_kernel<<<dim3((Skv + 3) / 4), dim3(256), 0, st>>>(bitmap, prefix, count, Skv, p.W);
-    key_scan_kernel<<<dim3(1), dim3(1024), 0, st>>>(count, start, Skv);
-    rank_kernel<<<dim3(2048), dim3(256), 0, st>>>(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, start, p.W, dstp);
+    order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
     bwd_pds_kernel<4><<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (const __bf16*)out,
                                                           (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);
@@ -704,7 +621,7 @@ extern "C" int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out
     first = false;
   }
   if (S == 0) {
-    zero_u32_kernel<<<dim3(256), dim3(256), 0, st>>>((unsigned*)acc, (size_t)Skv * DQK);
+    order::zero_u32_kernel<<<dim3(256), dim3(256), 0, st>>>((unsigned*)acc, (size_t)Skv * DQK);
   }
   cast_bf16_kernel<<<dim3(2048), dim3(256), 0, st>>>(acc, (unsigned short*)dkv, (size_t)Skv * DQK);
   DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(cast)");
