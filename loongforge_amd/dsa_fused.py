@@ -1,0 +1,336 @@
+"""Fused DeepSeek-Sparse-Attention modules with the reference's class names and signatures.
+
+Counterpart of loongforge/models/common/experimental_attention_variant/dsa_fused.py for one GPU:
+``DSAIndexerFused`` (:111) computes indexer q / k / weights and calls ``DSAIndexerKernel``;
+``DSAttentionFused`` (:718) runs indexer -> sparse attention -> sparse KL indexer loss.  The
+tensor-parallel all-to-alls of the reference are identities at tensor-parallel size 1 and are not
+present; sequence-chunked pipelining ("chunkpipe") is not supported.  The names
+``MegatronModule``, ``RotaryEmbedding``, ``DSAIndexerKernel`` and ``build_module`` are module
+attributes, as in the reference, so tests can patch them.
+"""
+import copy
+import math
+from dataclasses import dataclass
+from typing import Optional, Tuple, Union
+
+import torch
+import torch.nn.functional as F
+
+from .dsa_fused_kernels import DSADotProductAttention, DSAIndexerKernel, triton_attn_dist
+from .megatron_compat import (
+    AttnMaskType,
+    DSAIndexerLossAutoScaler,
+    DSAIndexerLossLoggingHelper as DSAIndexerLossLoggingHelperFused,
+    MegatronModule,
+    ModuleSpec,
+    PackedSeqParams,
+    ProcessGroupCollection,
+    RotaryEmbedding,
+    apply_rotary_pos_emb,
+    build_module,
+    get_args,
+    get_dsa_index_share_topk_holder,
+    is_dsa_skip_topk_layer,
+    source_dsa_compute_layer,
+)
+
+_HADAMARD_CACHE = {}
+
+
+def _hadamard(n: int, device, dtype):
+    key = (n, str(device), dtype)
+    if key not in _HADAMARD_CACHE:
+        assert n & (n - 1) == 0, "Hadamard size must be a power of two"
+        h = torch.ones(1, 1, dtype=torch.float32)
+        while h.shape[0] < n:
+            h = torch.cat([torch.cat([h, h], 1), torch.cat([h, -h], 1)], 0)
+        _HADAMARD_CACHE[key] = h.to(device=device, dtype=dtype)
+    return _HADAMARD_CACHE[key]
+
+
+def rotate_activation(x: torch.Tensor) -> torch.Tensor:
+    """Hadamard rotation of the last dimension scaled by ``dim ** -0.5`` (dsa_fused.py:74-90)."""
+    assert x.dtype == torch.bfloat16, f"rotate_activation only support bf16 input, but got {x.dtype}"
+    hidden_size = x.size(-1)
+    h = _hadamard(hidden_size, x.device, torch.float32)
+    return ((x.float() @ h) * hidden_size ** -0.5).to(x.dtype)
+
+
+@dataclass
+class DSAIndexerFusedSubmodules:
+    """Submodules of the indexer: query expansion, key projection, key norm, head-weight projection."""
+
+    linear_wq_b: Union[ModuleSpec, type] = None
+    linear_wk: Union[ModuleSpec, type] = None
+    k_norm: Union[ModuleSpec, type] = None
+    linear_weights_proj: Union[ModuleSpec, type] = None
+
+
+class DSAIndexerFused(MegatronModule):
+    """Lightning indexer: scores keys per query and returns the top-k (dsa_fused.py:111-703)."""
+
+    def __init__(self, config, submodules: DSAIndexerFusedSubmodules,
+                 pg_collection: Optional[ProcessGroupCollection] = None) -> None:
+        if not getattr(config, "dsa_indexer_use_sparse_loss", True):
+            raise ValueError(
+                "fused DSA only supports dsa_indexer_use_sparse_loss=True; "
+                "use portable DSA for dense indexer loss"
+            )
+        super().__init__(config=config)
+        self.hidden_size = self.config.hidden_size
+        self.qk_pos_emb_head_dim = self.config.qk_pos_emb_head_dim
+        self.q_lora_rank = (
+            self.config.q_lora_rank if self.config.q_lora_rank is not None else self.config.hidden_size
+        )
+        self.index_n_heads = self.config.dsa_indexer_n_heads
+        self.index_head_dim = self.config.dsa_indexer_head_dim
+        self.index_topk = self.config.dsa_indexer_topk
+        self.softmax_scale: float = self.index_head_dim ** -0.5
+
+        if pg_collection is None:
+            pg_collection = ProcessGroupCollection.use_mpu_process_groups(required_pgs=["tp", "cp", "pp"])
+        self.pg_collection = pg_collection
+
+        if self.config.rope_type == "rope":
+            self.rotary_pos_emb = RotaryEmbedding(
+                self.qk_pos_emb_head_dim,
+                rotary_percent=self.config.rotary_percent,
+                rotary_base=self.config.rotary_base,
+                cp_group=self.pg_collection.cp,
+            )
+        else:
+            raise ValueError(
+                f'Unsupported RoPE type: {self.config.rope_type}, supported types are "rope" and '
+                f'"yarn"'
+            )
+
+        self.linear_wq_b = build_module(
+            submodules.linear_wq_b,
+            self.q_lora_rank,
+            self.index_n_heads * self.index_head_dim,
+            config=self.config,
+            init_method=self.config.init_method,
+            bias=False,
+            skip_bias_add=False,
+            skip_weight_param_allocation=False,
+            parallel_mode="duplicated",
+        )
+        self.linear_wk = build_module(
+            submodules.linear_wk,
+            self.hidden_size,
+            self.index_head_dim,
+            config=self.config,
+            init_method=self.config.init_method,
+            bias=False,
+            skip_bias_add=False,
+            skip_weight_param_allocation=False,
+            parallel_mode="duplicated",
+        )
+        k_norm_config = copy.copy(self.config)
+        k_norm_config.normalization = "LayerNorm"
+        k_norm_eps = getattr(self.config, "dsa_indexer_k_norm_epsilon", None)
+        if k_norm_eps is None:
+            k_norm_eps = self.config.layernorm_epsilon
+        self.k_norm = build_module(
+            submodules.k_norm,
+            config=k_norm_config,
+            hidden_size=self.index_head_dim,
+            eps=k_norm_eps,
+        )
+        self.linear_weights_proj = build_module(
+            submodules.linear_weights_proj,
+            self.hidden_size,
+            self.index_n_heads,
+            config=self.config,
+            init_method=self.config.init_method,
+            bias=False,
+            skip_bias_add=False,
+            skip_weight_param_allocation=False,
+            parallel_mode="duplicated",
+        )
+        if getattr(self.config, "enable_chunkpipe", False):
+            raise NotImplementedError("chunkpipe is not supported by the single-GPU DSA modules")
+        self.indexer_kernel = DSAIndexerKernel()
+
+    def _apply_rope(self, x, rotary_pos_emb, mscale, cu_seqlens):
+        """RoPE on the leading ``qk_pos_emb_head_dim`` channels ("PE first", dsa_fused.py:453-487)."""
+        x_pe, x_nope = torch.split(
+            x, [self.qk_pos_emb_head_dim, self.index_head_dim - self.qk_pos_emb_head_dim], dim=-1
+        )
+        indexer_rope_config = copy.copy(self.config)
+        indexer_rope_config.multi_latent_attention = getattr(self.config, "dsa_indexer_rope_interleaved", False)
+        x_pe = apply_rotary_pos_emb(x_pe, rotary_pos_emb, config=indexer_rope_config, cu_seqlens=cu_seqlens,
+                                    mscale=mscale, cp_group=self.pg_collection.cp)
+        return torch.cat([x_pe, x_nope], dim=-1)
+
+    def get_query_key_weight_tensors(self, x, qr, packed_seq_params: Optional[PackedSeqParams] = None):
+        """q ``[s, (b,) h, d]``, k ``[s, (b,) d]``, weights ``[s, (b,) h]`` (dsa_fused.py:490-638)."""
+        x = x.detach()
+        qr = qr.detach()
+        rotary_seq_len = self.rotary_pos_emb.get_rotary_seq_len(None, None, x, self.config, packed_seq_params)
+        packed_seq = packed_seq_params is not None and packed_seq_params.qkv_format == "thd"
+        rotary_pos_emb = self.rotary_pos_emb(rotary_seq_len, offset=0, packed_seq=packed_seq)
+        mscale = 1.0
+        if packed_seq_params is not None:
+            cu_seqlens_q = packed_seq_params.cu_seqlens_q_padded
+            if cu_seqlens_q is None:
+                cu_seqlens_q = packed_seq_params.cu_seqlens_q
+            cu_seqlens_kv = packed_seq_params.cu_seqlens_kv_padded
+            if cu_seqlens_kv is None:
+                cu_seqlens_kv = packed_seq_params.cu_seqlens_kv
+        else:
+            cu_seqlens_q = cu_seqlens_kv = None
+
+        q, _ = self.linear_wq_b(qr)
+        q = q.view(*q.size()[:-1], self.index_n_heads, self.index_head_dim)
+        q = self._apply_rope(q, rotary_pos_emb, mscale, cu_seqlens_q)
+
+        k, _ = self.linear_wk(x)
+        k = self.k_norm(k)
+        if packed_seq_params is None:
+            k = k.unsqueeze(-2)
+            k = self._apply_rope(k, rotary_pos_emb, mscale, cu_seqlens_kv)
+            k = k.squeeze(-2)
+        else:
+            k = self._apply_rope(k.unsqueeze(-2), rotary_pos_emb, mscale, cu_seqlens_kv).squeeze(-2)
+
+        if getattr(self.config, "dsa_indexer_rotate_activation", True):
+            q = rotate_activation(q)
+            k = rotate_activation(k)
+
+        weights, _ = self.linear_weights_proj(x)
+        weights = weights * self.index_n_heads ** -0.5
+        return q, k, weights
+
+    def forward(self, x, qr, packed_seq_params: Optional[PackedSeqParams] = None):
+        """-> ``(index_score_topk [s, topk], topk_indices [s, topk])`` (dsa_fused.py:640-703)."""
+        indexer_query, indexer_key, indexer_weights = self.get_query_key_weight_tensors(x, qr, packed_seq_params)
+        if packed_seq_params is None:
+            indexer_query = indexer_query.squeeze(1).contiguous()
+        indexer_key = indexer_key.squeeze(1).contiguous()
+        indexer_weights = indexer_weights.squeeze(1).contiguous()
+        kv_offset = self.pg_collection.tp.rank() * indexer_query.size(0)
+        return self.indexer_kernel(
+            indexer_query,
+            indexer_key,
+            indexer_weights,
+            self.index_topk,
+            chunk_offset=kv_offset,
+            packed_seq_params=packed_seq_params,
+        )
+
+
+@dataclass
+class DSAttentionFusedSubmodules:
+    """Submodules of the sparse attention: the indexer."""
+
+    indexer: Union[ModuleSpec, type] = None
+
+
+class DSAttentionFused(MegatronModule):
+    """Indexer -> top-k -> sparse MLA attention -> sparse KL indexer loss (dsa_fused.py:718-971)."""
+
+    def __init__(self, config, submodules: DSAttentionFusedSubmodules, layer_number: int,
+                 attn_mask_type: AttnMaskType, attention_type: str, attention_dropout: Optional[float] = None,
+                 softmax_scale: Optional[float] = None, k_channels: Optional[int] = None,
+                 v_channels: Optional[int] = None, cp_comm_type: str = "p2p",
+                 pg_collection: ProcessGroupCollection = None, is_mtp_layer: bool = False):
+        super().__init__(config=config)
+        self.layer_number = layer_number
+        if is_mtp_layer:
+            self.layer_number = self.layer_number + self.config.num_layers
+        if pg_collection is None:
+            pg_collection = ProcessGroupCollection.use_mpu_process_groups(required_pgs=["tp", "cp", "pp"])
+        self.pg_collection = pg_collection
+        args = get_args()
+        self.use_dsa_sp_first = getattr(args, "use_dsa_sp_first", False) if args is not None else False
+
+        self.index_topk_freq = getattr(self.config, "dsa_indexer_topk_freq", 1)
+        self.index_skip_topk_offset = getattr(self.config, "dsa_indexer_skip_topk_offset", 0)
+        self.index_share = self.index_topk_freq > 1
+        self.skip_topk = (
+            self.index_share
+            and not is_mtp_layer
+            and is_dsa_skip_topk_layer(self.layer_number, self.index_skip_topk_offset, self.index_topk_freq)
+        )
+        self.source_layer = (
+            source_dsa_compute_layer(self.layer_number, self.index_skip_topk_offset, self.index_topk_freq)
+            if self.skip_topk
+            else self.layer_number
+        )
+        self.indexer = None
+        if not self.skip_topk:
+            self.indexer = build_module(submodules.indexer, config=self.config, pg_collection=pg_collection)
+
+        if softmax_scale is None:
+            softmax_scale = 1.0 / math.sqrt(k_channels if k_channels is not None else config.kv_channels)
+        self.softmax_scale = softmax_scale
+        self.sparse_attention = build_module(DSADotProductAttention, config=self.config,
+                                             softmax_scale=self.softmax_scale)
+        self.attn_sink = None
+        _DSA_MIN_HEAD_DIM = 128  # head count the sparse attention kernel is tiled for
+        self.num_attention_heads_padded = max(config.num_attention_heads, _DSA_MIN_HEAD_DIM)
+        self.num_attention_heads = config.num_attention_heads
+
+    def forward(self, query, key, value, attention_mask, x, qr, attn_mask_type: AttnMaskType = None,
+                attention_bias=None, packed_seq_params: PackedSeqParams = None, index_share_carrier: object = None):
+        """query ``[sq, b, h, 576]`` (or ``[t, h, 576]`` packed), key ``[skv, b, 576]`` -> ``[b, sq, h, 512]``
+        (``[t, h, 512]`` packed), with the indexer loss attached in training mode."""
+        sq = query.size(0)
+        topk_holder = (
+            get_dsa_index_share_topk_holder(packed_seq_params, index_share_carrier, self.skip_topk,
+                                            self.layer_number, self.source_layer)
+            if self.index_share
+            else None
+        )
+        if self.skip_topk:
+            if self.source_layer not in topk_holder:
+                raise RuntimeError(
+                    "DSA index-share skip layer "
+                    f"(layer_number={self.layer_number}) needs top-k indices from source "
+                    f"computing layer {self.source_layer}, but that layer did not run before it."
+                )
+            index_scores = None
+            topk_indices = topk_holder[self.source_layer]
+        else:
+            x = x.detach()
+            qr = qr.detach()
+            index_scores, topk_indices = self.indexer(x, qr, packed_seq_params=packed_seq_params)
+        if topk_holder is not None and not self.skip_topk:
+            topk_holder[self.layer_number] = topk_indices
+
+        chunk_query = query
+        if self.num_attention_heads < self.num_attention_heads_padded:
+            pad_size = self.num_attention_heads_padded - self.num_attention_heads
+            chunk_query = F.pad(chunk_query, [0, 0, 0, pad_size])
+        offset = self.pg_collection.tp.rank() * chunk_query.size(0)
+
+        output, p_out = self.sparse_attention(
+            chunk_query,
+            key,
+            topk_indices.unsqueeze(0).int(),
+            offset,
+            attn_mask_type=attn_mask_type,
+            packed_seq_params=packed_seq_params,
+            return_p_out=True,
+            attn_sink=self.attn_sink,
+        )
+        if self.num_attention_heads < self.num_attention_heads_padded:
+            output = output[..., : self.num_attention_heads, :]
+            p_out = p_out[:, : self.num_attention_heads, :]
+
+        if self.training and torch.is_grad_enabled() and not self.skip_topk:
+            indexer_loss_coeff = getattr(self.config, "dsa_indexer_loss_coeff", 0.0)
+            with torch.no_grad():
+                main_attn_probs = triton_attn_dist(p_out, self.softmax_scale)[:, : index_scores.shape[-1]]
+            index_attn_probs = torch.softmax(index_scores, dim=-1)
+            loss = F.kl_div((index_attn_probs + 1e-10).log(), main_attn_probs.float() + 1e-10, reduction="sum")
+            indexer_loss = indexer_loss_coeff * loss / sq
+            if indexer_loss_coeff > 0:
+                DSAIndexerLossLoggingHelperFused.save_loss_to_tracker(
+                    loss=indexer_loss,
+                    layer_number=self.layer_number,
+                    num_layers=self.config.num_layers + getattr(self.config, "mtp_num_layers", 0),
+                )
+            output = DSAIndexerLossAutoScaler.apply(output, indexer_loss)
+        return output

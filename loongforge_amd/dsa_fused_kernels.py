@@ -1,0 +1,249 @@
+"""Kernel wrappers of the fused DSA path, with the reference's names and call signatures.
+
+Drop-in counterparts of loongforge/models/common/experimental_attention_variant/dsa_fused_kernels.py
+(``triton_attn_dist`` :1898, ``padded_flashinfer_topk`` :1958, ``DSADotProductAttentionFunction``
+:2001, ``DSADotProductAttention`` :2115, ``DSAIndexerKernelFunction`` :2287, ``DSAIndexerKernel``
+:2445), backed by the gfx950 HIP kernels instead of DeepGEMM / FlashInfer / FlashMLA / Triton.
+"""
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from . import ops
+from .megatron_compat import AttnMaskType, MegatronModule, PackedSeqParams
+
+_LOG2E = 1.44269504
+
+
+def triton_attn_dist(p_out: torch.Tensor, sm_scale) -> torch.Tensor:
+    """``output[s, :] = mean_h softmax(p_out[s, h, :] * sm_scale)``.
+
+    Same contract as the reference function of this name (dsa_fused_kernels.py:1898-1955): input
+    ``(s_q, h_q, topk)``, output ``(s_q, topk)`` in ``p_out.dtype``, softmax in fp32.  The slot count
+    does not have to be a power of two here.
+    """
+    if p_out.ndim != 3:
+        raise ValueError("p_out must be (s_q, h_q, topk)")
+    return ops.attn_dist(p_out, float(sm_scale)).to(p_out.dtype)
+
+
+def padded_flashinfer_topk(logits, topk, sk, *, sorted=True):
+    """Top-k values and indices of the last dimension, padded when ``topk`` exceeds it.
+
+    Reference: dsa_fused_kernels.py:1958-1998.  Values come back descending when ``sorted``; when
+    ``topk > d`` the tail is filled with ``-inf`` / ``sk``.  Rows with fewer than ``topk`` finite
+    entries return id ``-1`` for the ``-inf`` slots (the reference leaves arbitrary masked ids there,
+    which its attention kernel rejects later; ``-1`` is rejected the same way).
+    """
+    d = logits.size(-1)
+    topk = int(topk)
+    lead = logits.shape[:-1]
+    flat = logits.reshape(-1, d).float()
+    k_eff = min(topk, d)
+    vals, idx = ops.topk(flat, k_eff, sorted=sorted)
+    if topk > d:
+        pad = topk - d
+        vals = torch.cat([vals, vals.new_full((vals.shape[0], pad), float("-inf"))], dim=-1)
+        idx = torch.cat([idx, idx.new_full((idx.shape[0], pad), sk)], dim=-1)
+    return vals.reshape(*lead, topk), idx.reshape(*lead, topk)
+
+
+class DSADotProductAttentionFunction(torch.autograd.Function):
+    """Sparse MLA attention over the selected latent rows (forward and backward on the HIP kernels).
+
+    Same argument list as the reference (dsa_fused_kernels.py:2006-2021).  ``topk_length``,
+    ``attn_sink`` and ``window_size`` belong to a different attention variant and must keep their
+    defaults.
+    """
+
+    @staticmethod
+    def forward(ctx, q, kv, indices, chunk_offset=0, sm_scale=None, d_v=512, return_p_out=False,
+                packed_seq_params=None, topk_length=None, attn_sink=None, window_size=0, fast_mode=False):
+        if topk_length is not None or attn_sink is not None or window_size not in (0, None):
+            raise NotImplementedError("topk_length / attn_sink / window_size are not supported by this build")
+        # q [sq, n, d]; kv [skv, 1, d]; indices [sq, 1, topk]
+        sq = q.size(0)
+        kv2 = kv.reshape(kv.shape[0], kv.shape[-1])
+        ids = indices.reshape(sq, indices.shape[-1])
+        out, lse, p_out = ops.sparse_mla_fwd(q, kv2, ids, chunk_offset, sm_scale, d_v, return_p_out)
+        ctx.save_for_backward(q, kv, ids, out, lse)
+        ctx.sm_scale = sm_scale
+        ctx.chunk_offset = chunk_offset
+        ctx.d_v = d_v
+        out = out.unsqueeze(0)
+        if return_p_out:
+            ctx.mark_non_differentiable(p_out)
+            return out, p_out
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out, grad_p_out=None):
+        q, kv, ids, out, lse = ctx.saved_tensors
+        grad_out = grad_out.squeeze(0).contiguous()
+        kv2 = kv.reshape(kv.shape[0], kv.shape[-1])
+        grad_q, grad_kv = ops.sparse_mla_bwd(q, kv2, out, grad_out, ids, lse, ctx.chunk_offset, ctx.sm_scale, ctx.d_v)
+        return (grad_q, grad_kv.reshape(kv.shape), None, None, None, None, None, None, None, None, None, None)
+
+
+class DSADotProductAttention(MegatronModule):
+    """Layout-normalising wrapper around the sparse attention kernel (dsa_fused_kernels.py:2115-2284)."""
+
+    def __init__(self, config, softmax_scale: Optional[float] = None):
+        super().__init__(config=config)
+        self.config = config
+        self.qkv_format: str = "sbhd"
+        self.softmax_scale = softmax_scale
+
+    def forward(self, query: Tensor, kv: Tensor, indices: Tensor, chunk_offset: int,
+                attn_mask_type: AttnMaskType = None, attention_bias: Tensor = None,
+                packed_seq_params: PackedSeqParams = None, return_p_out: bool = False, window_size: int = 0,
+                topk_length: Optional[Tensor] = None, attn_sink: Optional[Tensor] = None):
+        if attn_mask_type is None:
+            attn_mask_type = AttnMaskType.causal
+        assert attn_mask_type in (AttnMaskType.causal, AttnMaskType.padding_causal), (
+            "DSADotProductAttention only support causal attention."
+            "Please use TEDotProductAttention instead."
+        )
+        assert attention_bias is None, "Attention bias is not supported for DSADotProductAttention."
+        assert self.config.qk_pos_emb_head_dim == 64, (
+            f"DSADotProductAttention only support qk_pos_emb_head_dim 64, but got {self.config.qk_pos_emb_head_dim}."
+        )
+        qkv_format = self.qkv_format
+        if getattr(self.config, "apply_rope_fusion", False):
+            qkv_format = "bshd"
+        if packed_seq_params is not None and getattr(packed_seq_params, "qkv_format", None):
+            qkv_format = packed_seq_params.qkv_format
+
+        if qkv_format == "bshd" and getattr(self.config, "apply_rope_fusion", False):
+            query = query.transpose(0, 1).contiguous()
+            kv = kv.unsqueeze(2).transpose(0, 1).contiguous()
+        elif qkv_format == "thd":
+            kv = kv.unsqueeze(1)
+        else:  # sbhd: query [sq, b, n, d], kv [skv, b, d]
+            query = query.transpose(0, 1).contiguous()
+            kv = kv.unsqueeze(2).transpose(0, 1).contiguous()
+
+        assert indices is not None, "DSADotProductAttention need topk_indices."
+        indices = indices.unsqueeze(1) if qkv_format == "thd" else indices.unsqueeze(2)
+        # the kernels take one sequence (or one packed batch) at a time
+        if query.ndim == 4:
+            assert query.size(0) == 1, "DSADotProductAttention does not support batched input"
+            query = query.squeeze(0)
+        if kv.ndim == 4:
+            kv = kv.squeeze(0)
+        # callers in thd mode hand [1, total_q, topk]; it is memory-identical to [total_q, 1, topk]
+        indices = indices.reshape(-1, 1, indices.shape[-1])
+
+        topk = indices.size(-1)
+        topk_aligned = ((topk + 63) // 64) * 64
+        if topk_aligned != topk:
+            indices = torch.nn.functional.pad(indices, (0, topk_aligned - topk), value=-1)
+
+        d_qk = query.size(-1)
+        d_v = self.config.v_head_dim if d_qk == self.config.v_head_dim else self.config.kv_lora_rank
+
+        res = DSADotProductAttentionFunction.apply(query, kv, indices, chunk_offset, self.softmax_scale, d_v,
+                                                   return_p_out, packed_seq_params, topk_length, attn_sink,
+                                                   window_size, True)
+        core_attn_out, p_out = (res if return_p_out else (res, None))
+        if qkv_format == "thd":
+            core_attn_out = core_attn_out.squeeze(0).contiguous()
+        else:
+            core_attn_out = core_attn_out.contiguous()
+        if return_p_out:
+            return core_attn_out, p_out
+        return core_attn_out
+
+
+def _unscale_indexer_grad(grad, scale_inv):
+    """``grad / scale_inv`` with rows sitting on the quantiser's epsilon floor forced to zero
+    (loongforge/models/foundation/deepseek_v4/deepseek_v4_csa.py:1525-1541)."""
+    epsilon_scale_floor = 2.0 ** -48 * 1.5
+    scale_inv = scale_inv.unsqueeze(-1)
+    usable = torch.isfinite(scale_inv) & (scale_inv > epsilon_scale_floor)
+    safe = torch.where(usable, scale_inv, torch.ones_like(scale_inv))
+    return (grad / safe).masked_fill(~usable.expand_as(grad), 0.0)
+
+
+def _pad_to(x: Tensor, size: int, dim: int) -> Tensor:
+    if x.shape[dim] == size:
+        return x
+    pad = [0, 0] * (x.ndim - 1 - dim % x.ndim) + [0, size - x.shape[dim]]
+    return torch.nn.functional.pad(x, pad)
+
+
+class DSAIndexerKernelFunction(torch.autograd.Function):
+    """fp8 lightning indexer: quantise -> windowed logits -> top-k, with the sparse backward.
+
+    Reference: dsa_fused_kernels.py:2287-2442.  Differences that do not change results: the logits
+    never leave the kernels' workspace, ids of rows with fewer than ``index_topk`` visible keys are
+    ``-1`` instead of arbitrary masked positions, and head counts / head dims below the kernel's
+    tile sizes are zero-padded (exact: padded heads carry zero weight, padded dims zero products).
+    """
+
+    sorted_output = True
+
+    @staticmethod
+    def forward(ctx, index_q: Tensor, index_k: Tensor, weights: Tensor, index_topk: int, chunk_offset: int,
+                packed_seq_params: Optional[PackedSeqParams]):
+        assert index_q.ndim == 3 and index_k.ndim == 2 and weights.ndim == 2
+        seq_q, head, dim = index_q.size()
+        seq_k, _dim = index_k.size()
+        assert dim == _dim, "Query and Key have diff dim."
+        assert dim <= 128, "Only support dim with size 128."
+        device = index_q.device
+        softmax_scale = dim ** -0.5
+
+        head_p = 32 if head <= 32 else 64
+        assert head <= 64, "the indexer kernel supports at most 64 heads"
+        q_p = _pad_to(_pad_to(index_q.to(torch.bfloat16), 128, 2), head_p, 1).contiguous()
+        k_p = _pad_to(index_k.to(torch.bfloat16), 128, 1).contiguous()
+        q_fp8, q_scale = ops.quant_rowwise_e4m3(q_p)
+        k_fp8, k_scale = ops.quant_rowwise_e4m3(k_p)
+
+        if packed_seq_params is None:
+            k_start = torch.zeros(seq_q, dtype=torch.int, device=device)
+        else:
+            cu = packed_seq_params.cu_seqlens_kv_padded
+            if cu is None:
+                cu = packed_seq_params.cu_seqlens_kv
+            cu = cu.to(device)
+            seqlens = cu[1:] - cu[:-1]
+            full_seq_ids = torch.repeat_interleave(torch.arange(len(seqlens), device=device, dtype=torch.int), seqlens)
+            local_seq_ids = full_seq_ids[chunk_offset:chunk_offset + seq_q]
+            k_start = cu[local_seq_ids.long()].int()
+        k_end = torch.arange(seq_q, dtype=torch.int, device=device) + chunk_offset + 1
+
+        weight_scaled = _pad_to(weights.float(), head_p, 1) * q_scale * softmax_scale
+        index_score_topk, topk_indices = ops.indexer_topk(q_fp8, weight_scaled, k_fp8, k_scale, k_start, k_end,
+                                                          index_topk, DSAIndexerKernelFunction.sorted_output)
+        ctx.softmax_scale = softmax_scale
+        ctx.index_topk = index_topk
+        ctx.shape = (head, dim)
+        ctx.in_dtypes = (index_q.dtype, index_k.dtype, weights.dtype)
+        ctx.save_for_backward(q_fp8, k_fp8, q_scale, k_scale, weight_scaled, topk_indices)
+        ctx.mark_non_differentiable(topk_indices)
+        return index_score_topk, topk_indices
+
+    @staticmethod
+    def backward(ctx, grad_score, grad_topk):
+        q_fp8, k_fp8, q_scale, k_scale, weight_scaled, topk_indices = ctx.saved_tensors
+        head, dim = ctx.shape
+        grad_score = torch.where(topk_indices >= 0, grad_score.float(), torch.zeros_like(grad_score, dtype=torch.float32))
+        d_q, d_k, d_weights = ops.indexer_bwd(grad_score.contiguous(), q_fp8, k_fp8, k_scale, weight_scaled,
+                                              topk_indices.int())
+        d_weights = d_weights * q_scale * ctx.softmax_scale
+        d_q = _unscale_indexer_grad(d_q, q_scale)
+        d_k = _unscale_indexer_grad(d_k, k_scale)
+        dq_t, dk_t, dw_t = ctx.in_dtypes
+        return (d_q[:, :head, :dim].to(dq_t), d_k[:, :dim].to(dk_t), d_weights[:, :head].to(dw_t), None, None, None)
+
+
+class DSAIndexerKernel(torch.nn.Module):
+    """``forward(index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params)`` ->
+    ``(index_score_topk [sq, topk] fp32, topk_indices [sq, topk] int32)``; reference
+    dsa_fused_kernels.py:2445-2474."""
+
+    def forward(self, index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params):
+        return DSAIndexerKernelFunction.apply(index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params)

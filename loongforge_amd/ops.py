@@ -1,0 +1,335 @@
+"""Tensor-level entry points of the gfx950 DSA kernels.
+
+Every function here checks its arguments, allocates outputs and workspaces with torch (the C
+library allocates nothing), and calls libdsa_hip.so through ctypes on the current HIP stream.
+The raw kernels are also registered as torch custom ops in the ``dsa::`` namespace so that they
+can be used from compiled graphs and carry fake-tensor shape functions.
+
+There is no CPU path and no fallback: tensors must live on a HIP device.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_FP8 = torch.float8_e4m3fn
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("DSA kernels need tensors on a HIP device; got a %s tensor" % t.device.type)
+
+
+def _c(t: torch.Tensor) -> torch.Tensor:
+    return t if t.is_contiguous() else t.contiguous()
+
+
+# --------------------------------------------------------------------------------------------
+# quantiser
+# --------------------------------------------------------------------------------------------
+@torch.library.custom_op("dsa::quant_rowwise_e4m3", mutates_args=())
+def _quant_op(x: torch.Tensor, eps: float, pow2: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    _need_gpu(x)
+    if x.dtype != torch.bfloat16:
+        raise ValueError("quant_rowwise_e4m3 expects bf16 input, got %s" % x.dtype)
+    x = _c(x)
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    x8 = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    scale_inv = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        _lib.check(lib.dsa_quant_rowwise_e4m3(x.data_ptr(), rows, cols, x8.data_ptr(), scale_inv.data_ptr(),
+                                              float(eps), int(pow2), _stream(x)), "dsa_quant_rowwise_e4m3")
+    return x8, scale_inv
+
+
+@_quant_op.register_fake
+def _(x, eps, pow2):
+    return x.new_empty(x.shape, dtype=torch.uint8), x.new_empty(x.shape[:-1], dtype=torch.float32)
+
+
+def quant_rowwise_e4m3(x: torch.Tensor, eps: float = 1e-12, pow2: bool = True):
+    """bf16 ``[..., 128]`` -> (float8_e4m3fn payload, fp32 ``scale_inv`` per row)."""
+    x8, scale_inv = _quant_op(x, eps, pow2)
+    return x8.view(_FP8), scale_inv
+
+
+def _as_u8(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype == _FP8:
+        return t.view(torch.uint8)
+    if t.dtype != torch.uint8:
+        raise ValueError("expected an fp8-e4m3 (or raw uint8) tensor, got %s" % t.dtype)
+    return t
+
+
+# --------------------------------------------------------------------------------------------
+# indexer forward
+# --------------------------------------------------------------------------------------------
+def _check_indexer(q8, q_w, k8, k_scale, ks, ke):
+    _need_gpu(q8, q_w, k8, k_scale, ks, ke)
+    if q8.ndim != 3 or k8.ndim != 2 or q_w.ndim != 2:
+        raise ValueError("indexer expects q8 [S,H,128], k8 [Sk,128], q_w [S,H]")
+    S, Hi, D = q8.shape
+    if D != 128 or k8.shape[1] != 128:
+        raise ValueError("Only support dim with size 128.")
+    if q_w.shape != (S, Hi) or k_scale.shape != (k8.shape[0],) or ks.shape != (S,) or ke.shape != (S,):
+        raise ValueError("indexer: inconsistent shapes")
+    return S, Hi, k8.shape[0]
+
+
+@torch.library.custom_op("dsa::indexer_logits", mutates_args=())
+def _indexer_logits_op(q8: torch.Tensor, q_w: torch.Tensor, k8: torch.Tensor, k_scale: torch.Tensor,
+                       ks: torch.Tensor, ke: torch.Tensor, width: int, relative: bool) -> torch.Tensor:
+    S, Hi, Sk = _check_indexer(q8, q_w, k8, k_scale, ks, ke)
+    q8, k8 = _c(_as_u8(q8)), _c(_as_u8(k8))
+    q_w, k_scale = _c(q_w.float()), _c(k_scale.float())
+    ks, ke = _c(ks.int()), _c(ke.int())
+    logits = torch.empty(S, width, dtype=torch.float32, device=q8.device)
+    lib = _lib.load()
+    with torch.cuda.device(q8.device):
+        _lib.check(lib.dsa_indexer_logits(q8.data_ptr(), q_w.data_ptr(), k8.data_ptr(), k_scale.data_ptr(),
+                                          ks.data_ptr(), ke.data_ptr(), S, Hi, Sk, logits.data_ptr(), width, width,
+                                          int(relative), _stream(q8)), "dsa_indexer_logits")
+    return logits
+
+
+@_indexer_logits_op.register_fake
+def _(q8, q_w, k8, k_scale, ks, ke, width, relative):
+    return q_w.new_empty(q8.shape[0], width, dtype=torch.float32)
+
+
+def indexer_logits(q8, q_w, k8, k_scale, ks, ke, width: Optional[int] = None, relative: bool = False):
+    """Dense ``[S, width]`` fp32 logits, -inf outside ``[ks, ke)`` (column ``j - ks`` if relative)."""
+    return _indexer_logits_op(q8, q_w, k8, k_scale, ks, ke, int(width if width is not None else k8.shape[0]),
+                              bool(relative))
+
+
+@torch.library.custom_op("dsa::topk", mutates_args=())
+def _topk_op(logits: torch.Tensor, K: int, row_begin: Optional[torch.Tensor], row_end: Optional[torch.Tensor],
+             id_base: Optional[torch.Tensor], sort: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    _need_gpu(logits, row_begin, row_end, id_base)
+    if logits.ndim != 2 or logits.dtype != torch.float32:
+        raise ValueError("topk expects a 2-D fp32 tensor")
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    S, width = logits.shape
+    rb = _c(row_begin.int()) if row_begin is not None else None
+    re = _c(row_end.int()) if row_end is not None else None
+    ib = _c(id_base.int()) if id_base is not None else None
+    scores = torch.empty(S, K, dtype=torch.float32, device=logits.device)
+    ids = torch.empty(S, K, dtype=torch.int32, device=logits.device)
+    lib = _lib.load()
+    with torch.cuda.device(logits.device):
+        _lib.check(lib.dsa_topk(logits.data_ptr(), S, logits.stride(0) if S > 0 else width,
+                                rb.data_ptr() if rb is not None else None, re.data_ptr() if re is not None else None,
+                                width, ib.data_ptr() if ib is not None else None, K, int(sort), scores.data_ptr(),
+                                ids.data_ptr(), _stream(logits)), "dsa_topk")
+    return scores, ids
+
+
+@_topk_op.register_fake
+def _(logits, K, row_begin, row_end, id_base, sort):
+    return logits.new_empty(logits.shape[0], K), logits.new_empty(logits.shape[0], K, dtype=torch.int32)
+
+
+def topk(logits, K: int, row_begin=None, row_end=None, id_base=None, sorted: bool = True):
+    """Per-row top-K (scores, int32 ids); unused slots are (-inf, -1)."""
+    return _topk_op(logits, int(K), row_begin, row_end, id_base, bool(sorted))
+
+
+@torch.library.custom_op("dsa::indexer_topk", mutates_args=())
+def _indexer_topk_op(q8: torch.Tensor, q_w: torch.Tensor, k8: torch.Tensor, k_scale: torch.Tensor, ks: torch.Tensor,
+                     ke: torch.Tensor, K: int, sort: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    S, Hi, Sk = _check_indexer(q8, q_w, k8, k_scale, ks, ke)
+    q8, k8 = _c(_as_u8(q8)), _c(_as_u8(k8))
+    q_w, k_scale = _c(q_w.float()), _c(k_scale.float())
+    ks, ke = _c(ks.int()), _c(ke.int())
+    scores = torch.empty(S, K, dtype=torch.float32, device=q8.device)
+    ids = torch.empty(S, K, dtype=torch.int32, device=q8.device)
+    lib = _lib.load()
+    nbytes = lib.dsa_indexer_topk_workspace_bytes(S, Sk, K)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=q8.device)
+    with torch.cuda.device(q8.device):
+        _lib.check(lib.dsa_indexer_topk_fwd(q8.data_ptr(), q_w.data_ptr(), k8.data_ptr(), k_scale.data_ptr(),
+                                            ks.data_ptr(), ke.data_ptr(), S, Hi, Sk, K, int(sort), scores.data_ptr(),
+                                            ids.data_ptr(), ws.data_ptr(), nbytes, _stream(q8)),
+                   "dsa_indexer_topk_fwd")
+    return scores, ids
+
+
+@_indexer_topk_op.register_fake
+def _(q8, q_w, k8, k_scale, ks, ke, K, sort):
+    return q_w.new_empty(q8.shape[0], K, dtype=torch.float32), q_w.new_empty(q8.shape[0], K, dtype=torch.int32)
+
+
+def indexer_topk(q8, q_w, k8, k_scale, ks, ke, K: int, sorted: bool = True):
+    """Fused logits + top-K: (scores [S,K] fp32, global key ids [S,K] int32, -1 padded)."""
+    return _indexer_topk_op(q8, q_w, k8, k_scale, ks, ke, int(K), bool(sorted))
+
+
+@torch.library.custom_op("dsa::indexer_bwd", mutates_args=())
+def _indexer_bwd_op(g: torch.Tensor, q8: torch.Tensor, k8: torch.Tensor, k_scale: torch.Tensor, q_w: torch.Tensor,
+                    ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _need_gpu(g, q8, k8, k_scale, q_w, ids)
+    S, Hi, D = q8.shape
+    Sk = k8.shape[0]
+    K = ids.shape[1]
+    if g.shape != ids.shape or ids.shape[0] != S:
+        raise ValueError("indexer_bwd: grad and ids must both be [S, K]")
+    Kp = (K + 127) // 128 * 128
+    g = g.float()
+    ids = ids.int()
+    if Kp != K:                       # slots are processed 128 at a time
+        g = torch.nn.functional.pad(g, (0, Kp - K), value=0.0)
+        ids = torch.nn.functional.pad(ids, (0, Kp - K), value=-1)
+    g, ids = _c(g), _c(ids)
+    q8, k8 = _c(_as_u8(q8)), _c(_as_u8(k8))
+    q_w, k_scale = _c(q_w.float()), _c(k_scale.float())
+    d_q8 = torch.empty(S, Hi, D, dtype=torch.float32, device=q8.device)
+    d_k8 = torch.empty(Sk, D, dtype=torch.float32, device=q8.device)
+    d_qw = torch.empty(S, Hi, dtype=torch.float32, device=q8.device)
+    lib = _lib.load()
+    nbytes = lib.dsa_indexer_bwd_workspace_bytes(S, Hi, Sk, Kp)
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q8.device)
+    with torch.cuda.device(q8.device):
+        _lib.check(lib.dsa_indexer_bwd(g.data_ptr(), q8.data_ptr(), k8.data_ptr(), k_scale.data_ptr(), q_w.data_ptr(),
+                                       ids.data_ptr(), S, Hi, Sk, Kp, d_q8.data_ptr(), d_k8.data_ptr(), d_qw.data_ptr(),
+                                       ws.data_ptr(), nbytes, _stream(q8)), "dsa_indexer_bwd")
+    return d_q8, d_k8, d_qw
+
+
+@_indexer_bwd_op.register_fake
+def _(g, q8, k8, k_scale, q_w, ids):
+    return (q_w.new_empty(q8.shape, dtype=torch.float32), q_w.new_empty(k8.shape, dtype=torch.float32),
+            q_w.new_empty(q_w.shape, dtype=torch.float32))
+
+
+def indexer_bwd(g, q8, k8, k_scale, q_w, ids):
+    """Gradients of the selected logits w.r.t. the fp8 payloads and the scaled weights (fp32)."""
+    return _indexer_bwd_op(g, q8, k8, k_scale, q_w, ids)
+
+
+# --------------------------------------------------------------------------------------------
+# sparse MLA
+# --------------------------------------------------------------------------------------------
+def _check_mla(q, kv, ids):
+    _need_gpu(q, kv, ids)
+    if q.ndim != 3 or kv.ndim != 2 or ids.ndim != 2:
+        raise ValueError("sparse MLA expects q [S,H,576], kv [Skv,576], ids [S,K]")
+    if q.dtype != torch.bfloat16 or kv.dtype != torch.bfloat16:
+        raise ValueError("sparse MLA expects bf16 q and kv")
+    if q.shape[-1] != 576 or kv.shape[-1] != 576:
+        raise ValueError("you should assign dim otherwise: d_qk must be 576 (512 latent + 64 rope)")
+    if ids.shape[0] != q.shape[0]:
+        raise ValueError("ids and q disagree on the number of queries")
+    if ids.shape[1] % 64 != 0:
+        raise ValueError("top-k must be padded to a multiple of 64 (pad ids with -1)")
+
+
+@torch.library.custom_op("dsa::sparse_mla_fwd", mutates_args=())
+def _mla_fwd_op(q: torch.Tensor, kv: torch.Tensor, ids: torch.Tensor, q_start: int, sm_scale: float, d_v: int,
+                p_out_mode: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _check_mla(q, kv, ids)
+    q, kv, ids = _c(q), _c(kv), _c(ids.int())
+    S, H, _ = q.shape
+    K = ids.shape[1]
+    out = torch.empty(S, H, d_v, dtype=torch.bfloat16, device=q.device)
+    lse = torch.empty(S, H, dtype=torch.float32, device=q.device)
+    if p_out_mode == 0:
+        p_out = torch.empty(0, dtype=torch.bfloat16, device=q.device)
+    else:
+        p_out = torch.empty(S, H, K, dtype=torch.float32 if p_out_mode == 2 else torch.bfloat16, device=q.device)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        _lib.check(lib.dsa_sparse_mla_fwd(q.data_ptr(), kv.data_ptr(), ids.data_ptr(), S, H, kv.shape[0], K,
+                                          int(q_start), float(sm_scale), int(d_v), out.data_ptr(), lse.data_ptr(),
+                                          p_out.data_ptr() if p_out_mode else None, int(p_out_mode == 2), _stream(q)),
+                   "dsa_sparse_mla_fwd")
+    return out, lse, p_out
+
+
+@_mla_fwd_op.register_fake
+def _(q, kv, ids, q_start, sm_scale, d_v, p_out_mode):
+    S, H, _ = q.shape
+    p = q.new_empty(0) if p_out_mode == 0 else q.new_empty(S, H, ids.shape[1], dtype=torch.float32 if p_out_mode == 2 else torch.bfloat16)
+    return q.new_empty(S, H, d_v), q.new_empty(S, H, dtype=torch.float32), p
+
+
+def sparse_mla_fwd(q, kv, ids, q_start: int = 0, sm_scale: Optional[float] = None, d_v: int = 512,
+                   return_p_out: bool = False, p_out_dtype: torch.dtype = torch.bfloat16):
+    """(out bf16 [S,H,d_v], natural-log lse fp32 [S,H], p_out or None)."""
+    if sm_scale is None:
+        sm_scale = q.shape[-1] ** -0.5
+    mode = 0 if not return_p_out else (2 if p_out_dtype == torch.float32 else 1)
+    out, lse, p_out = _mla_fwd_op(q, kv, ids, int(q_start), float(sm_scale), int(d_v), mode)
+    return out, lse, (p_out if return_p_out else None)
+
+
+@torch.library.custom_op("dsa::sparse_mla_bwd", mutates_args=())
+def _mla_bwd_op(q: torch.Tensor, kv: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, ids: torch.Tensor,
+                lse: torch.Tensor, q_start: int, sm_scale: float, d_v: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    _check_mla(q, kv, ids)
+    _need_gpu(out, dout, lse)
+    q, kv, ids = _c(q), _c(kv), _c(ids.int())
+    out, dout, lse = _c(out), _c(dout.to(torch.bfloat16)), _c(lse.float())
+    S, H, _ = q.shape
+    K = ids.shape[1]
+    if out.shape != (S, H, d_v) or dout.shape != (S, H, d_v) or lse.shape != (S, H):
+        raise ValueError("sparse_mla_bwd: out/dout must be [S,H,d_v] and lse [S,H]")
+    dq = torch.empty_like(q)
+    dkv = torch.empty_like(kv)
+    lib = _lib.load()
+    nbytes = lib.dsa_sparse_mla_bwd_workspace_bytes(S, H, kv.shape[0], K)
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.check(lib.dsa_sparse_mla_bwd(q.data_ptr(), kv.data_ptr(), out.data_ptr(), dout.data_ptr(), ids.data_ptr(),
+                                          lse.data_ptr(), S, H, kv.shape[0], K, int(q_start), float(sm_scale),
+                                          int(d_v), dq.data_ptr(), dkv.data_ptr(), ws.data_ptr(), nbytes, _stream(q)),
+                   "dsa_sparse_mla_bwd")
+    return dq, dkv
+
+
+@_mla_bwd_op.register_fake
+def _(q, kv, out, dout, ids, lse, q_start, sm_scale, d_v):
+    return torch.empty_like(q), torch.empty_like(kv)
+
+
+def sparse_mla_bwd(q, kv, out, dout, ids, lse, q_start: int = 0, sm_scale: Optional[float] = None, d_v: int = 512):
+    """(dq, dkv) in bf16; dkv is accumulated in a fixed order (bit-reproducible)."""
+    if sm_scale is None:
+        sm_scale = q.shape[-1] ** -0.5
+    return _mla_bwd_op(q, kv, out, dout, ids, lse, int(q_start), float(sm_scale), int(d_v))
+
+
+@torch.library.custom_op("dsa::attn_dist", mutates_args=())
+def _attn_dist_op(p_out: torch.Tensor, sm_scale: float) -> torch.Tensor:
+    _need_gpu(p_out)
+    if p_out.ndim != 3 or p_out.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("attn_dist expects p_out [S,H,K] in bf16 or fp32")
+    if p_out.stride(2) != 1:
+        p_out = p_out.contiguous()
+    S, H, K = p_out.shape
+    target = torch.empty(S, K, dtype=torch.float32, device=p_out.device)
+    lib = _lib.load()
+    with torch.cuda.device(p_out.device):
+        _lib.check(lib.dsa_attn_dist(p_out.data_ptr(), int(p_out.dtype == torch.float32), S, H, K,
+                                     p_out.stride(0) if S > 0 else H * K, p_out.stride(1), float(sm_scale),
+                                     target.data_ptr(), _stream(p_out)), "dsa_attn_dist")
+    return target
+
+
+@_attn_dist_op.register_fake
+def _(p_out, sm_scale):
+    return p_out.new_empty(p_out.shape[0], p_out.shape[2], dtype=torch.float32)
+
+
+def attn_dist(p_out, sm_scale: float):
+    """fp32 ``[S,K]``: mean over heads of softmax over slots of ``p_out * sm_scale``."""
+    return _attn_dist_op(p_out, float(sm_scale))

@@ -1,0 +1,144 @@
+"""GPU parity: quantiser, indexer logits, top-k (through the C ABI via loongforge_amd.ops)."""
+import pytest
+import torch
+
+from oracle import dsa_oracle as O
+from tests.gpu_util import valid_sets_equal_up_to_noise
+
+pytestmark = pytest.mark.gpu
+
+
+def _quant_pair(iq, ik, dev):
+    from loongforge_amd import ops
+
+    q8, qs = ops.quant_rowwise_e4m3(iq.to(dev))
+    k8, ks = ops.quant_rowwise_e4m3(ik.to(dev))
+    return q8, qs, k8, ks
+
+
+def test_quantiser_is_bit_exact(gpu):
+    from loongforge_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(2000, 128, generator=g) * torch.logspace(-10, 6, 2000).unsqueeze(-1)).to(torch.bfloat16)
+    x[7] = 0
+    x[8, 0] = 3.5            # amax exactly on a power-of-two boundary of 448/amax
+    x[9, 0] = 3.515625
+    x[10, 3] = float(torch.finfo(torch.bfloat16).max)
+    r8, rs = O.quant_rowwise_e4m3(x)
+    x8, si = ops.quant_rowwise_e4m3(x.to(gpu))
+    assert torch.equal(x8.view(torch.uint8).cpu(), r8.view(torch.uint8))
+    assert torch.equal(si.cpu(), rs)
+    assert si[7].item() == 2.0 ** -48
+    # 3-D input (tokens, heads, 128) quantises per (token, head) row
+    y = torch.randn(33, 5, 128, generator=g).to(torch.bfloat16)
+    y8, ys = ops.quant_rowwise_e4m3(y.to(gpu))
+    r8, rs = O.quant_rowwise_e4m3(y)
+    assert ys.shape == (33, 5) and torch.equal(y8.view(torch.uint8).cpu(), r8.view(torch.uint8)) and torch.equal(ys.cpu(), rs)
+    with pytest.raises(ValueError):
+        ops.quant_rowwise_e4m3(torch.zeros(4, 64, dtype=torch.bfloat16, device=gpu))
+
+
+@pytest.mark.parametrize("S,Hi,K,cu,seed", [
+    (200, 64, 64, None, 42),
+    (333, 32, 128, None, 5),
+    (512, 64, 64, [0, 100, 101, 300, 512], 9),
+    (70, 64, 128, None, 11),          # every row has fewer than K visible keys
+])
+def test_logits_and_topk_against_oracle(gpu, S, Hi, K, cu, seed):
+    from loongforge_amd import ops
+
+    cu_t = torch.tensor(cu, dtype=torch.int32) if cu else None
+    iq, ik, w = O.make_indexer_inputs(S, Hi, 128, seed=seed)
+    sc_ref, idx_ref, aux = O.indexer_forward(iq, ik, w, K, 0, cu_t, dtype=torch.float64)
+    q8, qs, k8, ksc = _quant_pair(iq, ik, gpu)
+    assert torch.equal(q8.view(torch.uint8).cpu(), aux["q8"].view(torch.uint8))
+    ws = (w.to(gpu) * qs * 128 ** -0.5).contiguous()
+    ks, ke = aux["ks"].to(gpu), aux["ke"].to(gpu)
+
+    logits = ops.indexer_logits(q8, ws, k8, ksc, ks, ke)
+    L, R = logits.cpu(), aux["logits"]
+    fin = torch.isfinite(R)
+    assert torch.equal(torch.isfinite(L), fin)                      # -inf exactly outside [ks, ke)
+    # 64 signed terms of magnitude ~|w'| * |q.k| cancel; fp32 noise is relative to the term size
+    noise = 1e-4 * R[fin].abs().max().item()
+    assert (L[fin].double() - R[fin]).abs().max().item() <= noise
+
+    for srt in (True, False):
+        sc, ids = ops.topk(logits, K, ks, ke, None, sorted=srt)
+        v2, _ = O.topk_select(L, K)                                  # library routine on the same logits
+        scc, idc = sc.cpu(), ids.cpu()
+        if srt:
+            assert torch.equal(scc, v2)
+        else:
+            assert torch.equal(torch.sort(scc, descending=True).values, v2)
+            big = torch.where(idc >= 0, idc, torch.full_like(idc, 1 << 30)).long()
+            assert (torch.diff(big, dim=1) >= 0).all()             # ascending column order
+        got = torch.where(idc >= 0, L.gather(1, idc.clamp(min=0).long()), torch.full_like(scc, float("-inf")))
+        assert torch.equal(got, scc)                                # slot t of scores and ids stay aligned
+        for i in range(S):
+            a = idc[i][idc[i] >= 0]
+            assert a.numel() == len(set(a.tolist())) == min(K, int(ke[i] - ks[i]))
+            assert (a >= int(ks[i])).all() and (a < int(ke[i])).all()
+
+    sc, ids = ops.indexer_topk(q8, ws, k8, ksc, ks, ke, K)
+    assert valid_sets_equal_up_to_noise(ids, idx_ref, R, band=2 * noise) == 0
+
+
+def test_topk_is_bit_exact_when_the_arithmetic_is_exact(gpu):
+    """Small-integer payloads, unit scales and power-of-two weights make every product and sum
+    exact in fp32, so the selected sets must equal the oracle's with no tolerance band (scores are
+    made distinct so that there are no ties at the boundary)."""
+    from loongforge_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    S, Hi, K = 300, 32, 64
+    q = torch.randint(-3, 4, (S, Hi, 128), generator=g).float()
+    k = torch.randint(-3, 4, (S, 128), generator=g).float()
+    w = torch.full((S, Hi), 2.0 ** -4)
+    k[:, 0] = 0
+    q8, k8 = q.to(torch.float8_e4m3fn), k.to(torch.float8_e4m3fn)
+    ksc = torch.ones(S) + torch.arange(S) * 2.0 ** -12              # distinct, exactly representable scales
+    ks, ke = O.indexer_window(S, 0)
+    R = O.indexer_logits(q8, w, k8, ksc, ks, ke, dtype=torch.float64)
+    L = ops.indexer_logits(q8.to(gpu), w.to(gpu), k8.to(gpu), ksc.to(gpu), ks.to(gpu), ke.to(gpu)).cpu()
+    fin = torch.isfinite(R)
+    assert torch.equal(L[fin].double(), R[fin])
+    sc, ids = ops.indexer_topk(q8.to(gpu), w.to(gpu), k8.to(gpu), ksc.to(gpu), ks.to(gpu), ke.to(gpu), K)
+    vref, iref = O.topk_select(R.float(), K)
+    assert torch.equal(sc.cpu(), vref)
+    for i in range(S):
+        row = vref[i][vref[i] > float("-inf")]
+        if row.numel() == K and (R[i, : i + 1] == row.min().item()).sum() > 1:
+            continue                                                # an exact tie at the K-th value
+        assert set(ids[i][ids[i] >= 0].tolist()) == set(iref[i][iref[i] >= 0].tolist())
+
+
+def test_padded_flashinfer_topk_wrapper(gpu):
+    from loongforge_amd.dsa_fused_kernels import padded_flashinfer_topk
+
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn(10, 20, generator=g)
+    vals, idx = padded_flashinfer_topk(logits.to(gpu), 5, 20)
+    rv, ri = torch.topk(logits, 5)
+    assert torch.equal(vals.cpu(), rv) and torch.equal(idx.cpu().long(), ri)
+    vals, idx = padded_flashinfer_topk(logits.to(gpu), 25, 20)
+    assert vals.shape == (10, 25) and torch.isinf(vals[:, 20:]).all() and (idx[:, 20:] == 20).all()
+    assert torch.equal(vals[:, :20].cpu(), torch.sort(logits, descending=True).values)
+
+
+def test_relative_layout_of_packed_logits(gpu):
+    from loongforge_amd import ops
+
+    cu = torch.tensor([0, 40, 41, 128], dtype=torch.int32)
+    iq, ik, w = O.make_indexer_inputs(128, 64, 128, seed=3)
+    _, _, aux = O.indexer_forward(iq, ik, w, 16, 0, cu)
+    q8, qs, k8, ksc = _quant_pair(iq, ik, gpu)
+    ws = (w.to(gpu) * qs * 128 ** -0.5).contiguous()
+    ks, ke = aux["ks"].to(gpu), aux["ke"].to(gpu)
+    dense = ops.indexer_logits(q8, ws, k8, ksc, ks, ke).cpu()
+    rel = ops.indexer_logits(q8, ws, k8, ksc, ks, ke, width=87, relative=True).cpu()
+    for i in range(128):
+        n = int(ke[i] - ks[i])
+        assert torch.equal(rel[i, :n], dense[i, int(ks[i]): int(ke[i])])
+        assert torch.isinf(rel[i, n:]).all()

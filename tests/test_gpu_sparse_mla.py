@@ -1,0 +1,155 @@
+"""GPU parity: sparse MLA forward / backward and the attention distribution."""
+import pytest
+import torch
+
+from oracle import dsa_oracle as O
+from tests.gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_fwd(inp, dev, q_start=0, p_out=False, p_dtype=torch.bfloat16):
+    from loongforge_amd import ops
+
+    return ops.sparse_mla_fwd(inp.q.to(dev), inp.kv.to(dev), inp.idx.to(dev), q_start, inp.sm_scale, 512, p_out, p_dtype)
+
+
+@pytest.mark.parametrize("S,H,K,q_start,skv,seed", [
+    (64, 128, 64, 0, None, 0),
+    (300, 128, 128, 17, None, 1),
+    (256, 64, 256, 0, None, 2),
+    (130, 32, 192, 5, 400, 3),
+])
+def test_forward_against_oracle(gpu, S, H, K, q_start, skv, seed):
+    inp = O.make_mla_inputs(S, H, K, seed=seed, skv=skv, q_start=q_start)
+    out, lse, _ = _run_fwd(inp, gpu, q_start)
+    ro, rl, _ = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, q_start, inp.sm_scale, 512)
+    assert_close(out, ro, "out")
+    assert (lse.cpu() - rl).abs().max().item() < 1e-4
+
+
+def test_forward_p_out_and_attn_dist(gpu):
+    from loongforge_amd import ops
+    from loongforge_amd.dsa_fused_kernels import triton_attn_dist
+
+    inp = O.make_mla_inputs(200, 128, 128, seed=4)
+    _, _, rp = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, 0, inp.sm_scale, 512)
+    for dt in (torch.float32, torch.bfloat16):
+        _, _, p = _run_fwd(inp, gpu, 0, True, dt)
+        assert p.dtype == dt and p.shape == (200, 128, 128)
+        fin = torch.isfinite(rp)
+        assert torch.equal(torch.isfinite(p.float().cpu()), fin)          # -inf exactly on invalid slots
+        tol = 2e-4 if dt == torch.float32 else 0.26                         # bf16 ulp of |logit| < 64
+        assert (p.float().cpu()[fin] - rp[fin]).abs().max().item() < tol
+        tgt = ops.attn_dist(p, inp.sm_scale)
+        ref = O.attn_dist(rp, inp.sm_scale)
+        assert (tgt.cpu() - ref).abs().max().item() < (1e-5 if dt == torch.float32 else 6e-3)
+        assert (tgt.sum(-1).cpu() - 1).abs().max().item() < 1e-4
+        # head-sliced view (what the attention module passes when it padded the heads)
+        tgt16 = ops.attn_dist(p[:, :16], inp.sm_scale)
+        ref16 = O.attn_dist(rp[:, :16], inp.sm_scale)
+        assert (tgt16.cpu() - ref16).abs().max().item() < (1e-5 if dt == torch.float32 else 6e-3)
+        assert triton_attn_dist(p, inp.sm_scale).dtype == dt
+
+
+def test_forward_invalid_ids_and_empty_rows(gpu):
+    inp = O.make_mla_inputs(96, 128, 64, seed=5, skv=120, q_start=10)
+    idx = inp.idx.clone()
+    idx[5, 0] = -1
+    idx[6, 1] = 120            # == s_kv
+    idx[7, 2] = 119            # in range but in the future of query 7
+    idx[8, :] = -1             # no valid slot at all
+    idx[9] = idx[9][torch.randperm(64, generator=torch.Generator().manual_seed(1))]   # padding in the middle
+    inp.idx = idx
+    out, lse, p = _run_fwd(inp, gpu, 10, True, torch.float32)
+    ro, rl, rp = O.sparse_mla_fwd(inp.q, inp.kv, idx, 10, inp.sm_scale, 512)
+    assert_close(out, ro, "out")
+    assert out[8].abs().max().item() == 0 and torch.isinf(lse[8]).all() and (lse[8] > 0).all()
+    m = torch.isfinite(rl)
+    assert (lse.cpu()[m] - rl[m]).abs().max().item() < 1e-4
+    assert torch.equal(torch.isfinite(p.cpu()), torch.isfinite(rp))
+
+
+def test_forward_survives_a_late_dominant_key(gpu):
+    """A key whose logit exceeds everything before it by far more than 2^64 forces the exact-max
+    pass; the result must still match the oracle."""
+    inp = O.make_mla_inputs(80, 128, 64, seed=6)
+    kv = inp.kv.clone().float()
+    kv[70] = inp.q[79, 0].float() * 40.0          # q.k ~ 40 * |q|^2 for query 79, head 0
+    inp.kv = kv.to(torch.bfloat16)
+    inp.idx[79, 63] = 70                            # visited in the last tile position
+    out, lse, _ = _run_fwd(inp, gpu)
+    ro, rl, _ = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, 0, inp.sm_scale, 512)
+    assert_close(out, ro, "out", atol=4e-2)         # |kv[70]| is ~40x larger than the other rows
+    assert (lse.cpu() - rl).abs().max().item() < 2e-2 * rl.abs().max().item() * 1e-2 + 1e-2
+
+
+def test_forward_slot_permutation_invariance(gpu):
+    inp = O.make_mla_inputs(100, 128, 128, seed=7)
+    out1, lse1, _ = _run_fwd(inp, gpu)
+    perm = torch.randperm(128, generator=torch.Generator().manual_seed(2))
+    inp.idx = inp.idx[:, perm].contiguous()
+    out2, lse2, _ = _run_fwd(inp, gpu)
+    assert (out1.float() - out2.float()).abs().max().item() < 2e-2
+    assert (lse1 - lse2).abs().max().item() < 1e-4
+
+
+@pytest.mark.parametrize("S,H,K,q_start,skv,seed", [
+    (64, 128, 64, 0, None, 0),
+    (200, 128, 128, 40, 300, 3),
+    (160, 64, 64, 0, None, 5),
+])
+def test_backward_against_oracle_and_deterministic(gpu, S, H, K, q_start, skv, seed):
+    from loongforge_amd import ops
+
+    inp = O.make_mla_inputs(S, H, K, seed=seed, skv=skv, q_start=q_start)
+    q, kv, idx, do = inp.q.to(gpu), inp.kv.to(gpu), inp.idx.to(gpu), inp.dout.to(gpu)
+    out, lse, _ = ops.sparse_mla_fwd(q, kv, idx, q_start, inp.sm_scale)
+    dq, dkv = ops.sparse_mla_bwd(q, kv, out, do, idx, lse, q_start, inp.sm_scale)
+    rdq, rdkv = O.sparse_mla_bwd(inp.q, inp.kv, inp.idx, inp.dout, q_start, inp.sm_scale, 512)
+    assert_close(dq, rdq, "dq", scale_aware=True)
+    assert_close(dkv, rdkv, "dkv", scale_aware=True)
+    dq2, dkv2 = ops.sparse_mla_bwd(q, kv, out, do, idx, lse, q_start, inp.sm_scale)
+    assert torch.equal(dq, dq2) and torch.equal(dkv, dkv2)          # bit-identical
+
+
+def test_backward_chunked_workspace_through_the_c_abi(gpu):
+    """A workspace too small for all queries at once makes the library walk the queries in chunks;
+    the result must not change."""
+    from loongforge_amd import _lib, ops
+
+    inp = O.make_mla_inputs(300, 128, 128, seed=7)
+    q, kv, idx, do = inp.q.to(gpu), inp.kv.to(gpu), inp.idx.to(gpu), inp.dout.to(gpu)
+    out, lse, _ = ops.sparse_mla_fwd(q, kv, idx, 0, inp.sm_scale)
+    dq1, dkv1 = ops.sparse_mla_bwd(q, kv, out, do, idx, lse, 0, inp.sm_scale)
+    lib = _lib.load()
+    small = lib.dsa_sparse_mla_bwd_workspace_bytes(100, 128, 300, 128)
+    ws = torch.empty(small, dtype=torch.uint8, device=gpu)
+    dq2, dkv2 = torch.empty_like(q), torch.empty_like(kv)
+    rc = lib.dsa_sparse_mla_bwd(q.data_ptr(), kv.data_ptr(), out.data_ptr(), do.data_ptr(), idx.data_ptr(),
+                                lse.data_ptr(), 300, 128, 300, 128, 0, inp.sm_scale, 512, dq2.data_ptr(),
+                                dkv2.data_ptr(), ws.data_ptr(), small, None)
+    assert rc == 0, lib.dsa_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(dq1, dq2)
+    assert (dkv1.float() - dkv2.float()).abs().max().item() <= 2 * 2.0 ** -8 * dkv1.float().abs().max().item()
+    tiny = torch.empty(1024, dtype=torch.uint8, device=gpu)
+    rc = lib.dsa_sparse_mla_bwd(q.data_ptr(), kv.data_ptr(), out.data_ptr(), do.data_ptr(), idx.data_ptr(),
+                                lse.data_ptr(), 300, 128, 300, 128, 0, inp.sm_scale, 512, dq2.data_ptr(),
+                                dkv2.data_ptr(), tiny.data_ptr(), 1024, None)
+    assert rc == -3 and b"workspace" in lib.dsa_last_error()
+
+
+def test_argument_errors(gpu):
+    from loongforge_amd import ops
+
+    q = torch.zeros(8, 128, 576, dtype=torch.bfloat16, device=gpu)
+    kv = torch.zeros(8, 576, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(ValueError, match="multiple of 64"):
+        ops.sparse_mla_fwd(q, kv, torch.zeros(8, 48, dtype=torch.int32, device=gpu))
+    with pytest.raises(ValueError, match="576"):
+        ops.sparse_mla_fwd(q[..., :512].contiguous(), kv, torch.zeros(8, 64, dtype=torch.int32, device=gpu))
+    with pytest.raises(ValueError, match="head count"):
+        ops.sparse_mla_fwd(q[:, :16].contiguous(), kv, torch.zeros(8, 64, dtype=torch.int32, device=gpu))
+    with pytest.raises(ValueError, match="d_v"):
+        ops.sparse_mla_fwd(q, kv, torch.zeros(8, 64, dtype=torch.int32, device=gpu), d_v=256)
