@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused DSA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one pass of the hot path at sequence length 8192 with all inputs resident in HBM:
+  * lightning indexer (fp8, 64 heads x 128) + causal top-k 2048        (benchmark config 2)
+  * sparse MLA forward + backward, 128 heads, d_qk 576, d_v 512, top-k 2048   (config 4)
+Prints ONE JSON line.  `value` is the sparse-MLA forward+backward rate in TFLOP/s (algorithmic
+flops: 2*H*(576+512) forward and 2*H*(3*576+2*512) backward per valid (query, key) pair, pairs =
+sum_q min(prefix_q, 2048)); the indexer + top-k rate in tokens/s is reported next to it.
+`roofline` describes the longest-running kernel of the step, timed live with HIP events;
+`cpu_baseline` is the CPU oracle (a PyTorch restatement of the reference's math) on a bounded
+sample of the same workload, on this box's host cores.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+S, H, K, HI = 8192, 128, 2048, 64
+DQK, DV = 576, 512
+PEAK_BF16 = 2500.0      # TFLOP/s, dense
+PEAK_FP8 = 5000.0
+
+
+def cpu_baseline(inp, iq, ik, w, n_queries=2048):
+    """Oracle timed on an evenly spaced sample of queries (gather formulation, fp32)."""
+    import torch
+
+    from oracle import dsa_oracle as O
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    sel = torch.linspace(0, S - 1, n_queries).long()
+    q, idx, do = inp.q[sel], inp.idx[sel], inp.dout[sel]
+    pairs = int((idx >= 0).sum())
+    t0 = time.time()
+    # q_start = S disables the positional test (the ids are already causal for their own rows)
+    O.sparse_mla_bwd(q, inp.kv, idx, do, S, inp.sm_scale, DV)       # forward + backward by autograd
+    t_mla = time.time() - t0
+    flops = 2.0 * H * (4 * DQK + 3 * DV) * pairs
+    t0 = time.time()
+    q8, qs = O.quant_rowwise_e4m3(iq[sel])
+    k8, ks8 = O.quant_rowwise_e4m3(ik)
+    wk, we = O.indexer_window(S, 0)
+    logits = O.indexer_logits(q8, w[sel] * qs * 128 ** -0.5, k8, ks8, wk[sel], we[sel])
+    O.topk_select(logits, K)
+    t_idx = time.time() - t0
+    return {
+        "value": round(flops / t_mla / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": "%d evenly spaced queries of the seq-8192 workload: sparse-MLA fwd+bwd through the PyTorch oracle "
+                  "(%.1f s); indexer+top-k on the same queries (%.1f s)" % (n_queries, t_mla, t_idx),
+        "indexer_topk_tokens_per_s": round(n_queries / t_idx, 1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from loongforge_amd import _lib, ops
+    from oracle import dsa_oracle as O
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        sys.exit(1)
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+
+    # ---- synthetic inputs (CPU RNG, then resident in HBM) ------------------------------------
+    inp = O.make_mla_inputs(S, H, K, seed=0)
+    iq, ik, w = O.make_indexer_inputs(S, HI, 128, seed=42)
+    pairs = int((inp.idx >= 0).sum())
+    vis = S * (S + 1) // 2
+    q, kv, idx, do = inp.q.to(dev), inp.kv.to(dev), inp.idx.to(dev), inp.dout.to(dev)
+    iq_d, ik_d, w_d = iq.to(dev), ik.to(dev), w.to(dev)
+    ks, ke = (t.to(dev) for t in O.indexer_window(S, 0))
+    flops_fwd = 2.0 * H * (DQK + DV) * pairs
+    flops_bwd = 2.0 * H * (3 * DQK + 2 * DV) * pairs
+    flops_idx = 2.0 * HI * 128 * vis
+
+    wsb = lib.dsa_sparse_mla_bwd_workspace_bytes(S, H, S, K)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
+    dq, dkv = torch.empty_like(q), torch.empty_like(kv)
+    out = torch.empty(S, H, DV, dtype=torch.bfloat16, device=dev)
+    lse = torch.empty(S, H, dtype=torch.float32, device=dev)
+    pass_ms = (ctypes.c_float * 5)()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def ev():
+        return torch.cuda.Event(enable_timing=True)
+
+    t_idx = t_fwd = t_bwd = 0.0
+    t_pass = [0.0] * 5
+    t_logits = t_topk = 0.0
+    wall = 0.0
+    for step in range(args.warmup + args.steps):
+        timed = step >= args.warmup
+        torch.cuda.synchronize()
+        t0 = time.time()
+        e = [ev() for _ in range(6)]
+        e[0].record()
+        q8, qs = ops.quant_rowwise_e4m3(iq_d)
+        k8, ksc = ops.quant_rowwise_e4m3(ik_d)
+        wsd = (w_d * qs * 128 ** -0.5).contiguous()
+        e[1].record()
+        sc, ids = ops.indexer_topk(q8, wsd, k8, ksc, ks, ke, K)
+        e[2].record()
+        _lib.check(lib.dsa_sparse_mla_fwd(q.data_ptr(), kv.data_ptr(), idx.data_ptr(), S, H, S, K, 0, inp.sm_scale, DV,
+                                          out.data_ptr(), lse.data_ptr(), None, 0, stream), "fwd")
+        e[3].record()
+        _lib.check(lib.dsa_sparse_mla_bwd_profile(q.data_ptr(), kv.data_ptr(), out.data_ptr(), do.data_ptr(),
+                                                  idx.data_ptr(), lse.data_ptr(), S, H, S, K, 0, inp.sm_scale, DV,
+                                                  dq.data_ptr(), dkv.data_ptr(), ws.data_ptr(), wsb, stream, pass_ms),
+                   "bwd")
+        e[4].record()
+        torch.cuda.synchronize()
+        if timed:
+            wall += time.time() - t0
+            t_idx += e[0].elapsed_time(e[2])
+            t_fwd += e[2].elapsed_time(e[3])
+            t_bwd += e[3].elapsed_time(e[4])
+            for i in range(5):
+                t_pass[i] += pass_ms[i]
+    n = args.steps
+    t_idx, t_fwd, t_bwd = t_idx / n, t_fwd / n, t_bwd / n
+    t_pass = [x / n for x in t_pass]
+    # separate timing of the two indexer kernels (logits with dense layout + top-k on it)
+    e0, e1, e2 = ev(), ev(), ev()
+    e0.record()
+    lg = ops.indexer_logits(q8, wsd, k8, ksc, ks, ke)
+    e1.record()
+    ops.topk(lg, K, ks, ke)
+    e2.record()
+    torch.cuda.synchronize()
+    t_logits, t_topk = e0.elapsed_time(e1), e1.elapsed_time(e2)
+
+    mla_tflops = (flops_fwd + flops_bwd) / ((t_fwd + t_bwd) * 1e-3) / 1e12
+    # ---- roofline of the longest-running kernel of the step ---------------------------------------
+    pass_names = ["order", "bwd_pds_kernel (S, dP -> P, dS)", "bwd_dq_kernel (dQ)", "bwd_dkv_kernel (dKV rows)",
+                  "bwd_reduce_kernel (ordered dKV sum)"]
+    pass_flops = [0.0, 2.0 * H * (DQK + DV) * pairs, 2.0 * H * DQK * pairs, 2.0 * H * (DQK + DV) * pairs, 0.0]
+    kernels = [("mla_fwd_kernel", t_fwd, flops_fwd)] + [(pass_names[i], t_pass[i], pass_flops[i]) for i in range(5)]
+    name, t_dom, f_dom = max(kernels, key=lambda k: k[1])
+    if f_dom > 0:
+        roofline = {"kernel": name, "bound": "mfma", "achieved": round(f_dom / (t_dom * 1e-3) / 1e12, 1),
+                    "peak": PEAK_BF16, "unit": "TFLOP/s", "traffic": None}
+    else:   # the ordered reduction streams the per-pair rows: 1156 bytes per pair in, 2304 per key out
+        byts = 1156.0 * pairs + 2304.0 * S
+        roofline = {"kernel": name, "bound": "hbm", "achieved": round(byts / (t_dom * 1e-3) / 1e9, 1), "peak": 8000.0,
+                    "unit": "GB/s", "traffic": None}
+    roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
+    roofline["avg_launch_ms"] = round(t_dom, 3)
+
+    result = {
+        "metric": "sparse-MLA fwd+bwd TFLOP/s + indexer/top-k tokens/s, seq 8K, 1 GPU",
+        "value": round(mla_tflops, 1),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(t_idx + t_fwd + t_bwd, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "sparse MLA fwd+bwd seq 8192, 128 heads, d_qk 576, d_v 512, top-k 2048 (config 4) "
+                               "+ fp8 lightning indexer 64x128 with causal top-k 2048 (config 2)",
+                   "pairs": pairs, "visible_pairs": vis},
+        "frac_of_bf16_mfma_peak": round(mla_tflops / PEAK_BF16, 4),
+        "mla_fwd_ms": round(t_fwd, 3), "mla_bwd_ms": round(t_bwd, 3),
+        "mla_fwd_tflops": round(flops_fwd / (t_fwd * 1e-3) / 1e12, 1),
+        "mla_bwd_tflops": round(flops_bwd / (t_bwd * 1e-3) / 1e12, 1),
+        "mla_bwd_pass_ms": {pass_names[i]: round(t_pass[i], 3) for i in range(5)},
+        "indexer_topk_ms": round(t_idx, 3),
+        "indexer_topk_tokens_per_s": round(S / (t_idx * 1e-3), 1),
+        "indexer_topk_fp8_tflops": round(flops_idx / (t_idx * 1e-3) / 1e12, 1),
+        "indexer_topk_frac_of_fp8_peak": round(flops_idx / (t_idx * 1e-3) / 1e12 / PEAK_FP8, 4),
+        "indexer_logits_ms": round(t_logits, 3), "topk_ms": round(t_topk, 3),
+        "topk_hbm_gbps": round((4.0 * vis + 8.0 * S * K) / (t_topk * 1e-3) / 1e9, 1),
+        "wall_s_per_step": round(wall / n, 4),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(inp, iq, ik, w)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

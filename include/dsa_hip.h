@@ -125,6 +125,19 @@ int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out, const voi
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Profiling variant of dsa_sparse_mla_bwd: same arguments and results, plus the time of each pass
+ * in milliseconds, measured with HIP events on `stream` and summed over query chunks:
+ *   pass_ms[0] key-sorted order   [1] P and dS   [2] dQ   [3] per-pair dKV rows   [4] ordered dKV reduce
+ * It creates and destroys HIP events and waits for the stream before returning, so it is for
+ * benchmarks only.  No counterpart in the reference (its kernels are timed with do_bench from
+ * Python, ops/tilelang_ops/sparse_mla_bwd.py:359-368).
+ */
+int dsa_sparse_mla_bwd_profile(const void* q, const void* kv, const void* out, const void* dout,
+                               const int32_t* ids, const float* lse, int S, int H, int Skv, int K,
+                               int q_start, float sm_scale, int d_v, void* dq, void* dkv,
+                               void* workspace, size_t workspace_bytes, void* stream, float* pass_ms);
+
+/*
  * Head-averaged attention distribution over the selected slots:
  *   target[i,t] = (1/H) sum_h softmax_t(p_out[i,h,:] * sm_scale)[t]
  * Replaces triton_attn_dist, dsa_fused_kernels.py:1844-1955.  `ld_s` / `ld_h` are the element

@@ -566,9 +566,9 @@ extern "C" size_t dsa_sparse_mla_bwd_workspace_bytes(int S, int H, int Skv, int 
   return make_plan(S, Skv, K, DEFAULT_BUDGET).total;
 }
 
-extern "C" int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out, const void* dout, const int32_t* ids,
-                                  const float* lse, int S, int H, int Skv, int K, int q_start, float sm_scale, int d_v,
-                                  void* dq, void* dkv, void* workspace, size_t workspace_bytes, void* stream) {
+static int bwd_impl(const void* q, const void* kv, const void* out, const void* dout, const int32_t* ids,
+                    const float* lse, int S, int H, int Skv, int K, int q_start, float sm_scale, int d_v,
+                    void* dq, void* dkv, void* workspace, size_t workspace_bytes, void* stream, float* pass_ms) {
   DSA_REQUIRE(d_v == DV, "dsa_sparse_mla_bwd: only d_v = 512 (d_qk = 576) is supported, got d_v = %d", d_v);
   DSA_REQUIRE(S >= 0 && Skv > 0, "dsa_sparse_mla_bwd: bad sequence sizes S=%d Skv=%d", S, Skv);
   DSA_REQUIRE(H > 0 && H <= 128 && H % 32 == 0, "dsa_sparse_mla_bwd: head count must be 32, 64, 96 or 128, got %d", H);
@@ -603,21 +603,38 @@ extern "C" int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out
       hipFuncSetAttribute((const void*)bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemC) != hipSuccess)
     DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_bwd: cannot reserve LDS");
 
+  // optional per-pass timing (profiling entry point only): events between the passes
+  hipEvent_t ev[6];
+  if (pass_ms) {
+    for (int i = 0; i < 5; i++) pass_ms[i] = 0.f;
+    for (int i = 0; i < 6; i++) if (hipEventCreate(&ev[i]) != hipSuccess) DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_bwd_profile: cannot create events");
+  }
+#define DSA_MARK(i) do { if (pass_ms) hipEventRecord(ev[i], st); } while (0)
   bool first = true;
   for (int q0 = 0; q0 < S; q0 += p.chunk) {
     const int cnt = S - q0 < p.chunk ? S - q0 : p.chunk;
+    DSA_MARK(0);
     order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
+    DSA_MARK(1);
     bwd_pds_kernel<4><<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (const __bf16*)out,
                                                           (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(P, dS)");
+    DSA_MARK(2);
     bwd_dq_kernel<3><<<dim3(cnt), dim3(256), smemB, st>>>((const __bf16*)kv, ids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ)");
+    DSA_MARK(3);
     bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, ids, pds, dstp, rows, row_scale, q0, cnt,
                                                        H, Skv, K, q_start, p.chunk * K);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV rows)");
+    DSA_MARK(4);
     bwd_reduce_kernel<<<dim3(Skv), dim3(288), 0, st>>>(rows, row_scale, start, acc, Skv, first ? 0 : 1);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV reduce)");
+    DSA_MARK(5);
+    if (pass_ms) {
+      hipEventSynchronize(ev[5]);
+      for (int i = 0; i < 5; i++) { float ms = 0.f; hipEventElapsedTime(&ms, ev[i], ev[i + 1]); pass_ms[i] += ms; }
+    }
     first = false;
   }
   if (S == 0) {
@@ -626,5 +643,23 @@ extern "C" int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out
   cast_bf16_kernel<<<dim3(2048), dim3(256), 0, st>>>(acc, (unsigned short*)dkv, (size_t)Skv * DQK);
   DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(cast)");
   (void)NT;
+  if (pass_ms) for (int i = 0; i < 6; i++) hipEventDestroy(ev[i]);
+#undef DSA_MARK
   return DSA_OK;
+}
+
+extern "C" int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out, const void* dout, const int32_t* ids,
+                                  const float* lse, int S, int H, int Skv, int K, int q_start, float sm_scale, int d_v,
+                                  void* dq, void* dkv, void* workspace, size_t workspace_bytes, void* stream) {
+  return bwd_impl(q, kv, out, dout, ids, lse, S, H, Skv, K, q_start, sm_scale, d_v, dq, dkv, workspace, workspace_bytes,
+                  stream, nullptr);
+}
+
+extern "C" int dsa_sparse_mla_bwd_profile(const void* q, const void* kv, const void* out, const void* dout,
+                                          const int32_t* ids, const float* lse, int S, int H, int Skv, int K, int q_start,
+                                          float sm_scale, int d_v, void* dq, void* dkv, void* workspace,
+                                          size_t workspace_bytes, void* stream, float* pass_ms) {
+  DSA_REQUIRE(pass_ms != nullptr, "dsa_sparse_mla_bwd_profile: pass_ms must point at 5 floats");
+  return bwd_impl(q, kv, out, dout, ids, lse, S, H, Skv, K, q_start, sm_scale, d_v, dq, dkv, workspace, workspace_bytes,
+                  stream, pass_ms);
 }
