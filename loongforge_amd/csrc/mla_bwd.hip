@@ -10,7 +10,7 @@
 //                              exact MFMA operand layout of pass C (16 KB per query and tile)
 //   pass B  (bwd_dq_kernel)    dQ^T += KV^T.dS^T, both operands by LDS transpose reads
 //   pass C  (bwd_dkv_kernel)   per-pair rows  dS^T.Q + P^T.dO  (sum over all 128 heads) -> one
-//                              16-bit block-floating-point row (int16 mantissas + one fp32 scale)
+//                              bf16 row of 576 values
 //                              in a pair buffer, at the position given by a key-sorted order
 //   pass D  (bwd_reduce_kernel) dKV[key] = sum of that key's rows, in ascending query order
 // The key-sorted order (pass 0) comes from a bitmap key x query, its row-wise prefix popcounts and
@@ -302,65 +302,90 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
 // row[key, d] = sum_h dS[h,key] Q[h,d] + (d < 512) sum_h P[h,key] dO[h,d], all 128 heads, as
 // row^T = X^T . coef with X = [Q; dO] (k = heads).  X^T is the register-resident operand: wave w
 // owns the 32-column d-tiles {w, w+4, w+8, w+12, w+16} (the last only for w < 2) and loads its
-// columns once per query through LDS transpose reads; the coefficient operand is the pass-A tile
-// read from LDS as stored.  The finished 32 x 576 fp32 tile is staged in LDS, each row is scaled
-// by 32767 / max|row| and written as one contiguous 1152-byte row of int16 (plus its fp32 scale)
-// to the row index of the key-sorted order: the rounding error of a row is 2^-16 of its largest
-// element, 128 times less than a bf16 row of the same size.
-constexpr int OUT_STRIDE = DQK * 4 + 16;     // fp32 staging row stride in bytes (bank spread)
+// columns once per query through LDS transpose reads.  The 16 coefficient operands of a tile
+// (pass-A layout, read from LDS as stored) also sit in registers, so a column tile is finished by
+// 16 (or 8) back-to-back MFMAs on one accumulator.  Everything else runs in the shadow of the
+// matrix pipe, a few instructions after each MFMA: while column tile c+1 accumulates, tile c is
+// rounded to bf16, transposed through a wave-private LDS strip and stored as 64-byte pieces of
+// its 32 rows at the positions of the key-sorted order; while the last column tile of a tile
+// accumulates, the coefficient registers are refilled for the next tile.  One barrier per tile
+// (the coefficient transfer is shared by the four waves); the per-pair rows are bf16.
+constexpr int DKV_COEF_STAGES = 3;           // coefficient tiles in the LDS ring
+constexpr int DKV_STRIP_STRIDE = 80;         // bytes per row of the wave-private transpose strip
+constexpr int DKV_STRIP_BYTES = BI * DKV_STRIP_STRIDE;
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
-__global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(
+__device__ __forceinline__ unsigned cvt_pk_bf16(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
+
+// NC = column tiles of this wave (5 for waves 0 and 1, else 4).
+template <int NC>
+__device__ __forceinline__ void dkv_body(
     const __bf16* __restrict__ q, const __bf16* __restrict__ dout, const int* __restrict__ ids,
     const unsigned char* __restrict__ pds, const int* __restrict__ dst, unsigned char* __restrict__ rows,
-    float* __restrict__ row_scale, int q0, int cnt, int H, int Skv, int K, int q_start, int dummy_row) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  // [2][PDS_TILE_BYTES] coefficient tiles | [32][OUT_STRIDE] staging | [4][8192] per-wave X staging |
-  // ids arrays | dst rows of the query [K] | row inverse scales [32]
+    int q0, int cnt, int H, int Skv, int K, int q_start, int dummy_row, unsigned char* smem) {
+  constexpr int CST = DKV_COEF_STAGES;
+  constexpr int NU = NC == 5 ? 9 : 8;          // units of 8 MFMAs per tile
+  // [CST][PDS_TILE_BYTES] coefficient ring, shared with the set-up's per-wave X staging [4][8192] |
+  // [4][DKV_STRIP_BYTES] transpose strips | ids arrays | dst rows of the query [K + 32]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, g = lane >> 5;
   const int ql = cnt - 1 - (int)blockIdx.x;
   const int qi = q0 + ql;
   const int NT = K / BI;
-  unsigned char* out_s = smem + 2 * PDS_TILE_BYTES;
-  unsigned char* xs = out_s + BI * OUT_STRIDE + wave * 8192;
-  int* idx_s = (int*)(out_s + BI * OUT_STRIDE + 4 * 8192);
+  unsigned char* xs = smem + wave * 8192;
+  unsigned char* strip = smem + CST * PDS_TILE_BYTES + wave * DKV_STRIP_BYTES;
+  int* idx_s = (int*)(smem + CST * PDS_TILE_BYTES + 4 * DKV_STRIP_BYTES);
   unsigned* tmask = (unsigned*)(idx_s + K);
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
   int* dst_s = ntile_s + 4;
-  float* inv_s = (float*)(dst_s + K);
-  for (int t = tid; t < K; t += 256) {
-    const int d = dst[(size_t)ql * K + t];
+  for (int t = tid; t < K + BI; t += 256) {
+    const int d = t < K ? dst[(size_t)ql * K + t] : -1;
     dst_s[t] = d >= 0 ? d : dummy_row;       // invalid slots land in a scratch row: the store count stays fixed
   }
   const int ntiles = stage_ids(ids, qi, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
   if (ntiles == 0) return;
 
-  // ---- X^T operands: xq[c][kk] / xo[c][kk], kk = 2*w' + s' over the 8 groups of 16 heads ------
-  const int ncol = wave < 2 ? 5 : 4;
-  bf16x8 xq[5][8], xo[4][8];
+  // ---- X^T operands: x?[c][kk], kk = 2*w' + s' over the 8 groups of 16 heads ------------------
+  // Q columns 0..3 and all dO columns live in accumulation registers (MFMA reads them there), the
+  // fifth Q column, the coefficients and the accumulators in architectural registers.
+  bf16x8 xqa[4][8], xqv[8], xo[4][8];
   {
     typedef short i16x8 __attribute__((ext_vector_type(8)));
     const int blk = lane >> 4, ii = lane & 15;
     // transpose read of a [128 heads][32 d] block (64-byte rows): lane points at head
     // 32w' + 8(2s'+t) + 4g + ii/4, d chunk 16*(blk&1) + 4*(ii&3)
     const unsigned xoff = (unsigned)((4 * g + (ii >> 2)) * 64 + (16 * (blk & 1) + 4 * (ii & 3)) * 2);
-#pragma unroll
-    for (int pass = 0; pass < 9; pass++) {
-      const bool isq = pass < 5;
-      const int ci = isq ? pass : pass - 5;
-      if (isq && ci >= ncol) continue;
-      const int c = wave + 4 * ci;                      // d-tile
+    constexpr int NP = NC + 4;                 // passes: Q column tiles, then dO column tiles
+    uint4 ld[3][8];                            // three passes of global loads in flight
+    auto pass_load = [&](int pass, uint4 (&dstv)[8]) {
+      const bool isq = pass < NC;
+      const int ci = isq ? pass : pass - NC;
+      const int c = wave + 4 * ci;
       const __bf16* src = isq ? q + (size_t)qi * H * DQK + 32 * c : dout + (size_t)qi * H * DV + 32 * c;
       const int stride = isq ? DQK : DV;
-      // stage rows of 64 bytes: lane covers head (lane/4 + 16*it), 16-byte piece lane%4
+      // rows of 64 bytes: lane covers head (lane/4 + 16*it), 16-byte piece lane%4
 #pragma unroll
       for (int it = 0; it < 8; it++) {
         const int hh = (lane >> 2) + 16 * it;
-        uint4 val = make_uint4(0, 0, 0, 0);
-        if (hh < H) val = *(const uint4*)(src + (size_t)hh * stride + (lane & 3) * 8);
-        *(uint4*)(xs + hh * 64 + (lane & 3) * 16) = val;
+        dstv[it] = make_uint4(0, 0, 0, 0);
+        if (hh < H) dstv[it] = *(const uint4*)(src + (size_t)hh * stride + (lane & 3) * 8);
       }
+    };
+    pass_load(0, ld[0]);
+    pass_load(1, ld[1]);
+    pass_load(2, ld[2]);
+#pragma unroll
+    for (int pass = 0; pass < NP; pass++) {
+      const bool isq = pass < NC;
+      const int ci = isq ? pass : pass - NC;
+#pragma unroll
+      for (int it = 0; it < 8; it++) *(uint4*)(xs + ((lane >> 2) + 16 * it) * 64 + (lane & 3) * 16) = ld[pass % 3][it];
+      if (pass + 3 < NP) pass_load(pass + 3, ld[pass % 3]);
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
       for (int kk = 0; kk < 8; kk++) {
@@ -368,110 +393,142 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(
         i16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, hb + xoff));
         i16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, hb + 8 * 64 + xoff));
         const bf16x8 val = __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
-        if (isq) xq[ci][kk] = val; else xo[ci][kk] = val;
+        if (!isq) xo[ci][kk] = val;
+        else if (ci < 4) xqa[ci][kk] = val;
+        else xqv[kk] = val;
       }
       __builtin_amdgcn_wave_barrier();
     }
 #pragma unroll
-    for (int ci = 0; ci < 5; ci++)
+    for (int kk = 0; kk < 8; kk++) {
 #pragma unroll
-      for (int kk = 0; kk < 8; kk++) asm volatile("" : "+v"(xq[ci][kk]));
+      for (int ci = 0; ci < 4; ci++) asm volatile("" : "+a"(xqa[ci][kk]));
+      if (NC == 5) asm volatile("" : "+v"(xqv[kk]));
 #pragma unroll
-    for (int ci = 0; ci < 4; ci++)
-#pragma unroll
-      for (int kk = 0; kk < 8; kk++) asm volatile("" : "+a"(xo[ci][kk]));
+      for (int ci = 0; ci < 4; ci++) asm volatile("" : "+a"(xo[ci][kk]));
+    }
   }
+  __syncthreads();                             // the X staging shares LDS with the coefficient ring
 
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
   auto issue = [&](int n) {
-    const unsigned lb = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)((n & 1) * PDS_TILE_BYTES + wave * 1024));
+    const unsigned lb = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)((n % CST) * PDS_TILE_BYTES + wave * 1024));
     const unsigned char* src = uniform_ptr(pds + ((size_t)ql * NT + tlist[n]) * PDS_TILE_BYTES);
 #pragma unroll
     for (int c = 0; c < 4; c++) dma16(lb + c * 4096, (unsigned)(c * 4096 + tid * 16), src);
   };
-  issue(0);
+  // Vector-memory operations retire in issue order, so "the transfer of tile t has landed" is a
+  // bound on the number of operations issued after it: `issued` counts every operation of this
+  // wave, mk_a / mk_b are the counts right after the transfers of the next two tiles.
+  int issued = 0, mk_a = 0, mk_b = 0;
+  auto issue_marked = [&](int n) {
+    if (n < ntiles) {
+      issue(n);
+      issued += 4;
+    }
+    return issued;
+  };
+  // coefficient chunk of k-step kk: [kind][kk][g][key r] 16 bytes
+  const unsigned coff = (unsigned)(g * 512 + r * 16);
+  bf16x8 cf[16];
+  issue_marked(0);
+  mk_a = issue_marked(1);
+  if (ntiles > 1) { DSA_WAIT_VMCNT(4); } else { DSA_WAIT_VMCNT(0); }
+  __syncthreads();
+  mk_b = issue_marked(2);
+#pragma unroll
+  for (int k = 0; k < 16; k++) cf[k] = *(const bf16x8*)(smem + k * 1024 + coff);
+
+  // copy-out state: the two 16-byte pieces of the column tile in flight and the row pointers
+  // (row of key it*16 + lane/4, piece lane%4, this wave's first column tile) of the current tile
+  const size_t lane_off = (size_t)(wave * 64 + (lane & 3) * 16);
+  unsigned char* rptr[2];
+  rptr[0] = rptr[1] = rows + (size_t)dummy_row * ROW_BYTES + lane_off;
+  uint4 piece[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  const unsigned strip_w = (unsigned)(r * DKV_STRIP_STRIDE + 8 * g);
+  const unsigned strip_r = (unsigned)((lane >> 2) * DKV_STRIP_STRIDE + (lane & 3) * 16);
+  f32x16 acc[5];
+#pragma unroll
+  for (int e = 0; e < 16; e++) acc[NC - 1][e] = 0.f;   // rounded (to the scratch row) before its first MFMA
+
+  // tasks of column tile ci, spread over MFMA slots: round + transpose-write (4 slots), read back
+  // the two pieces (2 slots), store them (2 slots of the following unit)
+  auto conv = [&](int ci, int j) {
+    uint2 w;
+    w.x = cvt_pk_bf16(acc[ci][4 * j], acc[ci][4 * j + 1]);
+    w.y = cvt_pk_bf16(acc[ci][4 * j + 2], acc[ci][4 * j + 3]);
+    *(uint2*)(strip + strip_w + 16 * j) = w;
+  };
+  auto piece_read = [&](int it) { piece[it] = *(const uint4*)(strip + strip_r + it * 16 * DKV_STRIP_STRIDE); };
+  auto piece_store = [&](int ci, int it) {
+    *(uint4*)(rptr[it] + ci * 256) = piece[it];
+    issued += 1;
+  };
+
   for (int n = 0; n < ntiles; n++) {
-    // issued after this tile's 4 transfers: the 9 row stores and the scale store of the previous tile
-    if (n > 0) { DSA_WAIT_VMCNT(10); } else { DSA_WAIT_VMCNT(0); }
-    __syncthreads();
-    if (n + 1 < ntiles) issue(n + 1);
-    const unsigned char* cb = smem + (n & 1) * PDS_TILE_BYTES;
     const int tile = tlist[n];
-    f32x16 acc[5];
-    // coefficient chunk of k-step kk: [kind][kk][g][key r] 16 bytes
-    const unsigned coff = (unsigned)(g * 512 + r * 16);
-    bf16x8 cf[2];
-    cf[0] = *(const bf16x8*)(cb + coff);
-    cf[1] = *(const bf16x8*)(cb + 1024 + coff);
-    __builtin_amdgcn_sched_barrier(0);
+    const int drow0 = dst_s[tile * BI + (lane >> 2)], drow1 = dst_s[tile * BI + 16 + (lane >> 2)];
+    const unsigned char* nb = smem + ((n + 1) % CST) * PDS_TILE_BYTES;   // next tile's coefficients
 #pragma unroll
-    for (int step = 0; step < 16; step++) {            // 0..7: dS with Q, 8..15: P with dO
-      const int kk = step & 7;
-#pragma unroll
-      for (int ci = 0; ci < 5; ci++) {
-        if (step < 8) {
-          if (ci < 4 || wave < 2) {
-            if (step == 0) mfma_a_vv_first(acc[ci], xq[ci][kk], cf[step & 1]);
-            else mfma_a_vv(acc[ci], xq[ci][kk], cf[step & 1]);
-          }
-        } else if (ci < 4) {
-          mfma_a_av(acc[ci], xo[ci][kk], cf[step & 1]);
-        }
+    for (int u = 0; u < NU; u++) {
+      const int ci = u < 8 ? u >> 1 : 4, half = u < 8 ? (u & 1) : 0;
+      // column tile finished one unit ago (rounded now) and two units ago (stored now)
+      const int p1 = (u + NU - 1) % NU, p2 = (u + NU - 2) % NU;
+      const int conv_ci = p1 == 8 ? 4 : ((p1 & 1) ? p1 >> 1 : -1);
+      const int store_ci = p2 == 8 ? 4 : ((p2 & 1) ? p2 >> 1 : -1);
+      const bool reload = half == 1 ? u == 7 : u == (NC == 5 ? 8 : 6);
+      if (u == 6) {
+        if (n + 1 < ntiles) wait_vmcnt_le(issued - mk_a);
+        __syncthreads();
+        mk_a = mk_b;
+        mk_b = issue_marked(n + CST);
       }
-      if (step + 2 < 16) cf[step & 1] = *(const bf16x8*)(cb + (step + 2) * 1024 + coff);
+      if (u == 2) {                            // all stores of the previous tile are issued
+        rptr[0] = rows + (size_t)drow0 * ROW_BYTES + lane_off;
+        rptr[1] = rows + (size_t)drow1 * ROW_BYTES + lane_off;
+      }
       __builtin_amdgcn_sched_barrier(0);
-    }
-    // accumulator e of a lane: d = 32c + 8*(e/4) + 4g + (e%4), key = lane & 31
 #pragma unroll
-    for (int ci = 0; ci < 5; ci++) {
-      if (ci == 4 && wave >= 2) continue;
-      mfma_done_a(acc[ci]);
-      const int c = wave + 4 * ci;
-      float* orow = (float*)(out_s + r * OUT_STRIDE) + 32 * c + 4 * g;
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const f32x4 w = {acc[ci][4 * j], acc[ci][4 * j + 1], acc[ci][4 * j + 2], acc[ci][4 * j + 3]};
-        *(f32x4*)(orow + 8 * j) = w;
+      for (int m = 0; m < 8; m++) {
+        const bf16x8 b = cf[half * 8 + m];
+        if (half == 1) {
+          mfma_v_av(acc[ci], xo[ci][m], b);
+        } else if (ci == 4) {
+          if (m == 0) mfma_v_vv_first(acc[4], xqv[m], b); else mfma_v_vv(acc[4], xqv[m], b);
+        } else {
+          if (m == 0) mfma_v_av_first(acc[ci], xqa[ci][m], b); else mfma_v_av(acc[ci], xqa[ci][m], b);
+        }
+        if (reload) cf[half * 8 + m] = *(const bf16x8*)(nb + (half * 8 + m) * 1024 + coff);
+        if (conv_ci >= 0 && m >= 2 && m < 6) conv(conv_ci, m - 2);
+        if (conv_ci >= 0 && m >= 6) piece_read(m - 6);
+        if (store_ci >= 0 && (m == 3 || m == 4)) piece_store(store_ci, m - 3);
+        __builtin_amdgcn_sched_barrier(0);
       }
-    }
-    __syncthreads();
-    {   // per-row scale: 8 threads per row, 72 elements each
-      const int row = tid >> 3, part = tid & 7;
-      const float* src = (const float*)(out_s + row * OUT_STRIDE) + part * 72;
-      float mx = 0.f;
-#pragma unroll
-      for (int e = 0; e < 72; e += 4) {
-        const f32x4 w = *(const f32x4*)(src + e);
-        mx = fmaxf(fmaxf(mx, fmaxf(fabsf(w[0]), fabsf(w[1]))), fmaxf(fabsf(w[2]), fabsf(w[3])));
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
-      const bool finite = mx > 0.f && mx < INFINITY;
-      if (part == 0) {
-        inv_s[row] = finite ? 32767.0f / mx : 0.f;
-        row_scale[dst_s[tile * BI + row]] = finite ? mx / 32767.0f : 0.f;
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int it = 0; it < 9; it++) {
-      const int id = it * 256 + tid;
-      const int key = id / 72, ch = id % 72;
-      const float inv = inv_s[key];
-      const float* src = (const float*)(out_s + key * OUT_STRIDE) + ch * 8;
-      const f32x4 lo4 = *(const f32x4*)src, hi4 = *(const f32x4*)(src + 4);
-      int qv[8];
-#pragma unroll
-      for (int e = 0; e < 4; e++) { qv[e] = __float2int_rn(lo4[e] * inv); qv[4 + e] = __float2int_rn(hi4[e] * inv); }
-      uint4 val;
-      val.x = (unsigned)(qv[0] & 0xffff) | ((unsigned)qv[1] << 16);
-      val.y = (unsigned)(qv[2] & 0xffff) | ((unsigned)qv[3] << 16);
-      val.z = (unsigned)(qv[4] & 0xffff) | ((unsigned)qv[5] << 16);
-      val.w = (unsigned)(qv[6] & 0xffff) | ((unsigned)qv[7] << 16);
-      *(uint4*)(rows + (size_t)dst_s[tile * BI + key] * ROW_BYTES + ch * 16) = val;
     }
   }
+  // ---- drain: the last tile's final column tiles -------------------------------------------------
+  if (NC == 5) {
+    piece_store(3, 0);
+    piece_store(3, 1);
+  }
+  mfma_done_v(acc[NC - 1]);
+#pragma unroll
+  for (int j = 0; j < 4; j++) conv(NC - 1, j);
+  piece_read(0);
+  piece_read(1);
+  piece_store(NC - 1, 0);
+  piece_store(NC - 1, 1);
+}
+
+__global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ dout, const int* __restrict__ ids,
+    const unsigned char* __restrict__ pds, const int* __restrict__ dst, unsigned char* __restrict__ rows,
+    int q0, int cnt, int H, int Skv, int K, int q_start, int dummy_row) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  // waves 0 and 1 own five column tiles, waves 2 and 3 four: two copies of the whole body, so that
+  // no branch sits between the MFMAs; every copy meets the same barriers
+  if (threadIdx.x < 128) dkv_body<5>(q, dout, ids, pds, dst, rows, q0, cnt, H, Skv, K, q_start, dummy_row, smem);
+  else dkv_body<4>(q, dout, ids, pds, dst, rows, q0, cnt, H, Skv, K, q_start, dummy_row, smem);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -480,9 +537,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(
 // One 288-thread workgroup per key: 72 column chunks of 8 elements x 4 row groups (row r of the
 // segment goes to group r % 4); the four partial sums are combined in a fixed order, so the result
 // depends only on the segment, never on scheduling.  Pure streaming reads of 1152-byte rows.
-__global__ __launch_bounds__(288) void bwd_reduce_kernel(const unsigned char* __restrict__ rows, const float* __restrict__ row_scale,
-                                                         const int* __restrict__ start, float* __restrict__ dkv_acc, int Skv,
-                                                         int accumulate) {
+__global__ __launch_bounds__(288) void bwd_reduce_kernel(const unsigned char* __restrict__ rows, const int* __restrict__ start,
+                                                         float* __restrict__ dkv_acc, int Skv, int accumulate) {
   __shared__ float part[4][DQK];
   const int key = blockIdx.x;
   const int ch = threadIdx.x % 72, grp = threadIdx.x / 72;
@@ -492,12 +548,11 @@ __global__ __launch_bounds__(288) void bwd_reduce_kernel(const unsigned char* __
   for (int e = 0; e < 8; e++) acc[e] = 0.f;
   for (int rr = s0 + grp; rr < s1; rr += 4) {
     const uint4 v = *(const uint4*)(rows + (size_t)rr * ROW_BYTES + ch * 16);
-    const float sc = row_scale[rr];
-    const int w[4] = {(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+    const unsigned w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-      acc[2 * e] = fmaf((float)((w[e] << 16) >> 16), sc, acc[2 * e]);
-      acc[2 * e + 1] = fmaf((float)(w[e] >> 16), sc, acc[2 * e + 1]);
+      acc[2 * e] += __builtin_bit_cast(float, w[e] << 16);
+      acc[2 * e + 1] += __builtin_bit_cast(float, w[e] & 0xffff0000u);
     }
   }
 #pragma unroll
@@ -521,7 +576,7 @@ __global__ void cast_bf16_kernel(const float* __restrict__ src, unsigned short* 
 struct BwdPlan {
   int chunk;            // queries per pass over the buffers
   int W;                // bitmap words per key
-  size_t off_bitmap, off_prefix, off_count, off_start, off_dst, off_pds, off_rows, off_scale, off_acc, total;
+  size_t off_bitmap, off_prefix, off_count, off_start, off_dst, off_pds, off_rows, off_acc, total;
 };
 
 size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -538,7 +593,6 @@ BwdPlan layout_plan(int chunk, int Skv, int K) {
   p.off_dst = o; o = align_up(o + (size_t)chunk * K * 4);
   p.off_pds = o; o = align_up(o + (size_t)chunk * (K / BI) * PDS_TILE_BYTES);
   p.off_rows = o; o = align_up(o + ((size_t)chunk * K + 1) * ROW_BYTES);
-  p.off_scale = o; o = align_up(o + ((size_t)chunk * K + 1) * 4);
   p.off_acc = o; o = align_up(o + (size_t)Skv * DQK * 4);
   p.total = o;
   return p;
@@ -591,13 +645,12 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   int* dstp = (int*)(ws + p.off_dst);
   unsigned char* pds = ws + p.off_pds;
   unsigned char* rows = ws + p.off_rows;
-  float* row_scale = (float*)(ws + p.off_scale);
   float* acc = (float*)(ws + p.off_acc);
   const int NT = K / BI;
 
   const size_t smemA = (size_t)4 * TILE_BYTES + ids_lds_bytes(K) + 16 + 1024;
   const size_t smemB = (size_t)3 * (TILE_BYTES + PDS_KIND_BYTES) + ids_lds_bytes(K);
-  const size_t smemC = (size_t)2 * PDS_TILE_BYTES + (size_t)BI * OUT_STRIDE + 4 * 8192 + ids_lds_bytes(K) + 16 + (size_t)K * 4 + 128;
+  const size_t smemC = (size_t)DKV_COEF_STAGES * PDS_TILE_BYTES + 4 * DKV_STRIP_BYTES + ids_lds_bytes(K) + 16 + (size_t)(K + BI) * 4;
   if (hipFuncSetAttribute((const void*)bwd_pds_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemA) != hipSuccess ||
       hipFuncSetAttribute((const void*)bwd_dq_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemB) != hipSuccess ||
       hipFuncSetAttribute((const void*)bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemC) != hipSuccess)
@@ -624,11 +677,11 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     bwd_dq_kernel<3><<<dim3(cnt), dim3(256), smemB, st>>>((const __bf16*)kv, ids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ)");
     DSA_MARK(3);
-    bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, ids, pds, dstp, rows, row_scale, q0, cnt,
+    bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, ids, pds, dstp, rows, q0, cnt,
                                                        H, Skv, K, q_start, p.chunk * K);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV rows)");
     DSA_MARK(4);
-    bwd_reduce_kernel<<<dim3(Skv), dim3(288), 0, st>>>(rows, row_scale, start, acc, Skv, first ? 0 : 1);
+    bwd_reduce_kernel<<<dim3(Skv), dim3(288), 0, st>>>(rows, start, acc, Skv, first ? 0 : 1);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV reduce)");
     DSA_MARK(5);
     if (pass_ms) {

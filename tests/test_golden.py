@@ -73,6 +73,7 @@ def test_kernels_match_indexer_fixture(gpu):
     noise = 1e-4 * np.abs(ref["logits_sample"]).max()
     assert np.abs(G.sample(logits.masked_fill(~fin, 0.0), 3, 3) - ref["logits_sample"]).max() <= noise
     sc, ids = ops.indexer_topk(q8, ws, k8, ksc, ks.to(gpu), ke.to(gpu), c["K"])
-    got = sc.cpu().masked_fill(~torch.isfinite(sc.cpu()), -1e30).double().numpy()
+    got = sc.cpu().double().numpy()
+    got = np.where(np.isfinite(got), got, -1e30)      # padded slots are stored as -1e30 in the fixture
     assert np.abs(got - ref["scores"]).max() <= noise
     assert np.array_equal(ids.cpu().numpy() >= 0, ref["ids"] >= 0)
