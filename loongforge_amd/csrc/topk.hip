@@ -67,6 +67,76 @@ __device__ __forceinline__ Pick pick_bin(const int* hist, int nb, int need, int*
   return p;
 }
 
+// Order of the sorted output: descending score, ascending id among equal scores (id -1 last).
+__device__ __forceinline__ bool comes_first(float a, int ia, float b, int ib) {
+  return (a > b) || (a == b && (unsigned)ia < (unsigned)ib);
+}
+
+// Bitonic sort of Kp2 = EPT * BLOCK (score, id) pairs held in LDS.  A pair becomes one 64-bit
+// key whose unsigned order is the output order (descending score, then ascending id, id -1 last),
+// so a compare-exchange is one 64-bit compare and two selects.  Thread t keeps
+// elements [t*EPT, (t+1)*EPT) in registers: strides below EPT are register compare-exchanges,
+// strides inside a wave's span exchange through LDS without a workgroup barrier (LDS operations
+// of one wave complete in order), and only the strides that cross waves need barriers.  The
+// exchange buffer holds element j of thread t at j * BLOCK + t, so every LDS access of a wave is
+// bank-conflict free; the sorted elements go straight from registers to global memory.
+__device__ __forceinline__ unsigned long long sort_key(float score, int id) {
+  const unsigned bits = __builtin_bit_cast(unsigned, score + 0.0f);          // -0 -> +0
+  const unsigned asc = bits ^ ((bits >> 31) ? 0xffffffffu : 0x80000000u);    // ascending with the score
+  return ((unsigned long long)(~asc) << 32) | (unsigned)id;
+}
+__device__ __forceinline__ float sort_key_score(unsigned long long key) {
+  const unsigned asc = ~(unsigned)(key >> 32);
+  return __builtin_bit_cast(float, asc ^ ((asc >> 31) ? 0x80000000u : 0xffffffffu));
+}
+
+template <int EPT>
+__device__ __forceinline__ void bitonic_regs(float* outv, int* outi, unsigned long long* xbuf, int Kp2, float* sv, int* si, int K) {
+  const int tid = threadIdx.x;
+  const int base = tid * EPT;
+  unsigned long long key[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; j++) key[j] = sort_key(outv[base + j], outi[base + j]);
+  __syncthreads();                             // the buffer is reused as the exchange buffer below
+  for (int size = 2; size <= Kp2; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      if (stride >= EPT) {
+        const int pt = tid ^ (stride / EPT);
+        const bool cross_wave = stride / EPT >= 64;
+#pragma unroll
+        for (int j = 0; j < EPT; j++) xbuf[j * BLOCK + tid] = key[j];
+        if (cross_wave) __syncthreads(); else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        unsigned long long pk[EPT];
+#pragma unroll
+        for (int j = 0; j < EPT; j++) pk[j] = xbuf[j * BLOCK + pt];
+        if (cross_wave) __syncthreads(); else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // this lane keeps the smaller key when it holds the lower element of an ascending pair or
+        // the upper element of a descending one (size > stride >= EPT: the same for all j)
+        const bool keep_small = ((base & stride) == 0) == ((base & size) == 0);
+#pragma unroll
+        for (int j = 0; j < EPT; j++) key[j] = ((key[j] < pk[j]) == keep_small) ? key[j] : pk[j];
+      } else {
+#pragma unroll
+        for (int st = EPT >> 1; st > 0; st >>= 1) {
+          if (st != stride) continue;
+#pragma unroll
+          for (int j = 0; j < EPT; j++) {
+            if (j & st) continue;
+            const bool asc = ((base + j) & size) == 0;
+            const unsigned long long x = key[j], y = key[j | st];
+            const bool x_first = (x < y) == asc;
+            key[j] = x_first ? x : y;
+            key[j | st] = x_first ? y : x;
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < EPT; j++)
+    if (base + j < K) { sv[base + j] = sort_key_score(key[j]); si[base + j] = (int)(unsigned)key[j]; }
+}
+
 template <bool STAGED>
 __global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ logits, long ld,
                                                      const int* __restrict__ row_begin, const int* __restrict__ row_end,
@@ -156,18 +226,26 @@ __global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ l
   __syncthreads();
 
   if (sorted) {   // bitonic sort, descending score, ascending id among equal scores
-    for (int size = 2; size <= Kp2; size <<= 1) {
-      for (int stride = size >> 1; stride > 0; stride >>= 1) {
-        for (int t = tid; t < (Kp2 >> 1); t += BLOCK) {
-          const int lo = 2 * t - (t & (stride - 1));
-          const int hi = lo + stride;
-          const bool desc = ((lo & size) == 0);
-          const float a = outv[lo], b = outv[hi];
-          const int ia = outi[lo], ib = outi[hi];
-          const bool a_first = (a > b) || (a == b && (unsigned)ia < (unsigned)ib);   // id -1 sorts last
-          if (a_first != desc) { outv[lo] = b; outv[hi] = a; outi[lo] = ib; outi[hi] = ia; }
+    const int ept = Kp2 / BLOCK;
+    if (ept == 8) { bitonic_regs<8>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
+    else if (ept == 4) { bitonic_regs<4>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
+    else if (ept == 2) { bitonic_regs<2>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
+    else if (ept == 1) { bitonic_regs<1>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
+    else if (ept == 16) { bitonic_regs<16>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
+    else if (ept == 32) { bitonic_regs<32>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
+    else {
+      for (int size = 2; size <= Kp2; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+          for (int t = tid; t < (Kp2 >> 1); t += BLOCK) {
+            const int lo = 2 * t - (t & (stride - 1));
+            const int hi = lo + stride;
+            const bool desc = ((lo & size) == 0);
+            const float a = outv[lo], b = outv[hi];
+            const int ia = outi[lo], ib = outi[hi];
+            if (comes_first(a, ia, b, ib) != desc) { outv[lo] = b; outv[hi] = a; outi[lo] = ib; outi[hi] = ia; }
+          }
+          __syncthreads();
         }
-        __syncthreads();
       }
     }
   }
