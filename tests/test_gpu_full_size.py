@@ -4,6 +4,7 @@ import pytest
 import torch
 
 from oracle import dsa_oracle as O
+from tests.test_gpu_indexer_bwd import _reference as _indexer_reference
 
 pytestmark = pytest.mark.gpu
 
@@ -96,3 +97,96 @@ def test_sparse_mla_full_size_forward_backward(gpu):
         # relative to the largest gradient, and the elementwise bound holds for all but a sliver
         assert d.max().item() <= 5e-3 * rdkv.abs().max().item()
         assert (d > 2e-2 + 1e-2 * rdkv.abs()).float().mean().item() < 1e-3
+
+
+def test_packed_32k_pipeline(gpu):
+    """Config 5: 32768 tokens in 4 packed documents through the whole path - fp8 indexer + per-document
+    causal top-2048, sparse MLA forward with logits, attn_dist, KL loss, indexer backward and sparse
+    MLA backward (chunked workspace) - checked on sampled queries against the oracle and through
+    linearity (gradients of a dO / grad that is zero outside the sample) and bit-determinism."""
+    from loongforge_amd import ops
+
+    T, H, Hi, K, DV = 32768, 128, 64, 2048, 512
+    cu = O.make_packed_cu_seqlens(T, 4, 2048, seed=7)
+    assert int(cu[-1]) == T
+    iq, ik, w = O.make_indexer_inputs(T, Hi, 128, seed=7)
+    ks, ke = O.indexer_window(T, 0, cu)
+    q8, qs = ops.quant_rowwise_e4m3(iq.to(gpu))
+    k8, ksc = ops.quant_rowwise_e4m3(ik.to(gpu))
+    ws = (w.to(gpu) * qs * 128 ** -0.5).contiguous()
+    ksd, ked = ks.to(gpu), ke.to(gpu)
+    sc, ids = ops.indexer_topk(q8, ws, k8, ksc, ksd, ked, K)
+    valid = ids >= 0
+    assert (valid.sum(-1) == torch.clamp(ked - ksd, max=K)).all()
+    assert (((ids >= ksd[:, None]) & (ids < ked[:, None])) | ~valid).all()      # inside the own document, causal
+    srt = torch.sort(ids, dim=1).values
+    assert ((srt[:, 1:] != srt[:, :-1]) | (srt[:, 1:] < 0)).all()
+
+    # sample: first / last tokens of documents, short and long prefixes
+    b = cu.tolist()
+    sel = torch.tensor(sorted({0, 1, b[1] - 1, b[1], b[1] + 5, b[2] + 2047, b[2] + 2048, b[3] - 1, b[3], T - 1}))
+    seld = sel.to(gpu)
+    R = O.indexer_logits(q8.cpu()[sel], ws.cpu()[sel], k8.cpu(), ksc.cpu(), ks[sel], ke[sel], dtype=torch.float64)
+    for n, i in enumerate(sel.tolist()):
+        a = set(ids[i][ids[i] >= 0].tolist())
+        fin = torch.isfinite(R[n])
+        top = torch.topk(R[n], min(K, int(fin.sum())))
+        band = 2e-4 * R[n][fin].abs().max().item()
+        assert all(abs(R[n, j].item() - top.values[-1].item()) <= band for j in a ^ set(top.indices.tolist()))
+
+    # ---- sparse MLA forward with logits, attn_dist ------------------------------------------------
+    g = torch.Generator(device=gpu).manual_seed(7)
+    q = torch.randn(T, H, 576, generator=g, device=gpu, dtype=torch.float32).to(torch.bfloat16)
+    kv = torch.randn(T, 576, generator=g, device=gpu, dtype=torch.float32).to(torch.bfloat16)
+    sm = 192.0 ** -0.5
+    out, lse, p_out = ops.sparse_mla_fwd(q, kv, ids, 0, sm, return_p_out=True)
+    qs_c, kv_c, ids_c = q[seld].cpu(), kv.cpu(), ids[seld].cpu()
+    ro, rl, rp = O.sparse_mla_fwd(qs_c, kv_c, ids_c, T, sm, DV)
+    assert (out[seld].float().cpu() - ro).abs().max().item() <= 2e-2
+    assert (lse[seld].cpu() - rl).abs().max().item() <= 1e-4
+    target = ops.attn_dist(p_out, sm)
+    rt = O.attn_dist(rp, sm)
+    assert (target[seld].cpu() - rt).abs().max().item() <= 2e-3
+    assert ((target.sum(-1) - 1.0).abs() <= 1e-3).all()
+    del p_out
+
+    # ---- KL loss on the selected scores and indexer backward --------------------------------------
+    scg = sc.detach().clone().requires_grad_(True)
+    loss = O.indexer_kl_loss(scg, target, 1.0, T)
+    loss.backward()
+    gs = torch.where(valid, scg.grad, torch.zeros_like(sc)).contiguous()
+    assert torch.isfinite(loss) and torch.isfinite(gs).all()
+    gm = torch.zeros_like(gs)
+    gm[seld] = gs[seld]
+    d_q8, d_k8, d_qw = ops.indexer_bwd(gm, q8, k8, ksc, ws, ids)
+    aux = {"q8": q8.cpu()[sel], "k8": k8.cpu(), "weight_scaled": ws.cpu()[sel], "k_scale": ksc.cpu()}
+    rq, rk, rw, amb_qh, amb_key = _indexer_reference(aux, ids_c, gs[seld].cpu(), noise=2.0 ** -16)   # a 128-term fp32 sum: (n-1) * 2^-24 = 2^-17
+    eq = (d_q8[seld].double().cpu() - rq).abs().masked_fill(amb_qh[..., None], 0)
+    ek = (d_k8.double().cpu() - rk).abs().masked_fill(amb_key[:, None], 0)
+    ew = (d_qw[seld].double().cpu() - rw).abs()
+    assert eq.max().item() <= 1e-4 * rq.abs().max().item()
+    assert ek.max().item() <= 1e-4 * rk.abs().max().item()
+    assert ew.max().item() <= 1e-4 * rw.abs().max().item()
+    rest = torch.ones(T, dtype=torch.bool, device=gpu)
+    rest[seld] = False
+    assert (d_q8[rest] == 0).all() and (d_qw[rest] == 0).all()
+
+    def close(a, r, what):
+        tol = max(2e-2, 5e-3 * r.abs().max().item())
+        err = (a.float().cpu() - r.float()).abs().max().item()
+        assert err <= tol, "%s: max abs error %.4g > %.4g (max |ref| %.4g)" % (what, err, tol, r.abs().max().item())
+
+    # ---- sparse MLA backward: sampled dQ, dKV by linearity, determinism ---------------------------
+    dout = torch.randn(T, H, DV, generator=g, device=gpu, dtype=torch.float32).to(torch.bfloat16)
+    dq, dkv = ops.sparse_mla_bwd(q, kv, out, dout, ids, lse, 0, sm)
+    dq2, dkv2 = ops.sparse_mla_bwd(q, kv, out, dout, ids, lse, 0, sm)
+    assert torch.equal(dq, dq2) and torch.equal(dkv, dkv2)
+    rdq, rdkv = O.sparse_mla_bwd(qs_c, kv_c, ids_c, dout[seld].cpu(), T, sm, DV)
+    # the stated tolerance, element by element: 2e-2 absolute plus 1e-2 relative
+    assert ((dq[seld].float().cpu() - rdq).abs() <= 2e-2 + 1e-2 * rdq.abs()).all()
+    dm = torch.zeros_like(dout)
+    dm[seld] = dout[seld]
+    dqm, dkvm = ops.sparse_mla_bwd(q, kv, out, dm, ids, lse, 0, sm)
+    close(dkvm, rdkv, "dKV of the sampled queries")
+    assert torch.equal(dqm[seld], dq[seld])
+    assert torch.isfinite(dkv.float()).all() and torch.isfinite(dq.float()).all()

@@ -7,7 +7,7 @@ from oracle import dsa_oracle as O
 pytestmark = pytest.mark.gpu
 
 
-def _reference(aux, idx, g):
+def _reference(aux, idx, g, noise=2.0 ** -18):
     """fp64 autograd through the gathered logits + the set of (query, head) rows / keys touched by a
     ReLU gate whose exact pre-activation is within fp32 accumulation noise of zero (there the gate
     may legitimately fall on either side)."""
@@ -21,7 +21,7 @@ def _reference(aux, idx, g):
     ksel = k8f.double()[safe]
     rex = torch.einsum("mhd,mkd->mhk", q8f.double(), ksel)
     mag = torch.einsum("mhd,mkd->mhk", q8f.double().abs(), ksel.abs())
-    amb = (rex.abs() <= 2.0 ** -18 * mag) & (idx >= 0)[:, None, :]
+    amb = (rex.abs() <= noise * mag) & (idx >= 0)[:, None, :]
     amb_key = torch.zeros(k8f.shape[0], dtype=torch.bool)
     amb_key[safe[amb.any(1)]] = True
     return qf.grad, kf.grad, wf.grad, amb.any(-1), amb_key
