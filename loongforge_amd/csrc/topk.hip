@@ -137,6 +137,125 @@ __device__ __forceinline__ void bitonic_regs(float* outv, int* outi, unsigned lo
     if (base + j < K) { sv[base + j] = sort_key_score(key[j]); si[base + j] = (int)(unsigned)key[j]; }
 }
 
+// Sorted top-K of a staged row in one sweep, for rows whose finite values spread over a range:
+// a histogram over HBINS equal-width value bins (bin 0 = largest values) finds the bin that holds
+// the K-th largest value; every element of a better bin, plus all elements of that bin, is
+// scattered into its bin's segment of an LDS buffer (a counting sort, segments in descending value
+// order), and each scattered element then finds its final position by counting the elements of its
+// own segment that precede it in the output order (descending score, ascending column).  Elements
+// of the threshold bin that rank beyond the K-th place are dropped.  The result is exact and does
+// not depend on the order in which the atomics land.  Returns false without writing anything when
+// the row is unsuitable (no spread, or a crowded bin): the caller then takes the general path.
+constexpr int LIN_SPARE = 1024;              // extra buffer entries for the threshold bin's surplus
+constexpr int LIN_MAX_BIN = 256;             // largest segment ranked by pairwise counting
+
+__device__ __forceinline__ bool linear_select_sort(const float* __restrict__ src, unsigned* keys, int n, int K, int base_id,
+                                                   int* hist, int* scratch, unsigned long long* obuf, float* sv, int* si) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // ---- stage the row as keys; range of the finite values ---------------------------------------
+  float mn = INFINITY, mx = -INFINITY;
+  int nfin = 0;
+  for (int e0 = tid; e0 < n; e0 += 8 * BLOCK) {   // eight loads in flight per thread
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = e0 + i * BLOCK < n ? src[e0 + i * BLOCK] : -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if (e0 + i * BLOCK < n) keys[e0 + i * BLOCK] = f2key(v[i]);
+      if (fabsf(v[i]) < INFINITY) { mn = fminf(mn, v[i]); mx = fmaxf(mx, v[i]); nfin++; }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    nfin += __shfl_xor(nfin, o, 64);
+  }
+  __syncthreads();
+  if (lane == 0) { ((float*)scratch)[wave] = mn; ((float*)scratch)[4 + wave] = mx; scratch[8 + wave] = nfin; }
+  __syncthreads();
+  mn = fminf(fminf(((float*)scratch)[0], ((float*)scratch)[1]), fminf(((float*)scratch)[2], ((float*)scratch)[3]));
+  mx = fmaxf(fmaxf(((float*)scratch)[4], ((float*)scratch)[5]), fmaxf(((float*)scratch)[6], ((float*)scratch)[7]));
+  nfin = scratch[8] + scratch[9] + scratch[10] + scratch[11];
+  __syncthreads();
+  const float span = mx - mn;
+  if (!(span > 0.f) || !(span < INFINITY)) return false;
+  const int keff = min(K, nfin);
+  const float scale = ((float)HBINS - 0.5f) / span;
+  auto bin_of = [&](float v) { return min(HBINS - 1, (int)((mx - v) * scale)); };
+  // ---- histogram ------------------------------------------------------------------------------
+  for (int b = tid; b < HBINS; b += BLOCK) hist[b] = 0;
+  __syncthreads();
+  for (int e = tid; e < n; e += BLOCK) {
+    const float v = key2f(keys[e]);
+    if (fabsf(v) < INFINITY) atomicAdd(&hist[bin_of(v)], 1);
+  }
+  __syncthreads();
+  // ---- threshold bin: thread t owns bins [16t, 16t + 16) -------------------------------------------
+  constexpr int PER = HBINS / BLOCK;
+  int cnt[PER], local = 0;
+#pragma unroll
+  for (int b4 = 0; b4 < PER; b4 += 4) {
+    const int4 q4 = *(const int4*)(hist + tid * PER + b4);
+    cnt[b4] = q4.x; cnt[b4 + 1] = q4.y; cnt[b4 + 2] = q4.z; cnt[b4 + 3] = q4.w;
+  }
+#pragma unroll
+  for (int b = 0; b < PER; b++) local += cnt[b];
+  int total;
+  const int before = block_exscan(local, scratch, total);
+  if (before < keff && before + local >= keff) {
+    int run = before;
+#pragma unroll
+    for (int b = 0; b < PER; b++) {
+      if (run < keff && run + cnt[b] >= keff) { scratch[8] = tid * PER + b; scratch[9] = run; scratch[10] = cnt[b]; }
+      run += cnt[b];
+    }
+  }
+  __syncthreads();
+  const int tbin = scratch[8], above = scratch[9], c = scratch[10];
+  int big = 0;
+#pragma unroll
+  for (int b = 0; b < PER; b++) if (tid * PER + b < tbin) big = max(big, cnt[b]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) big = max(big, __shfl_xor(big, o, 64));
+  __syncthreads();
+  if (lane == 0) scratch[wave] = big;
+  __syncthreads();
+  big = max(max(scratch[0], scratch[1]), max(scratch[2], scratch[3]));
+  if (big > LIN_MAX_BIN || c > LIN_SPARE) return false;
+  // ---- segment starts (in place), scatter -------------------------------------------------------
+  {
+    int run = before, st[PER];
+#pragma unroll
+    for (int b = 0; b < PER; b++) { st[b] = run; run += cnt[b]; }
+#pragma unroll
+    for (int b4 = 0; b4 < PER; b4 += 4) *(int4*)(hist + tid * PER + b4) = make_int4(st[b4], st[b4 + 1], st[b4 + 2], st[b4 + 3]);
+  }
+  __syncthreads();
+  for (int e = tid; e < n; e += BLOCK) {
+    const float v = key2f(keys[e]);
+    if (fabsf(v) < INFINITY) {
+      const int b = bin_of(v);
+      if (b <= tbin) obuf[atomicAdd(&hist[b], 1)] = sort_key(v, e);
+    }
+  }
+  __syncthreads();
+  // ---- rank inside the segment: hist[b] is now the end of segment b ------------------------------
+  const int filled = above + c;
+  for (int p = tid; p < filled; p += BLOCK) {
+    const unsigned long long key = obuf[p];
+    const float v = sort_key_score(key);
+    const int b = bin_of(v);
+    const int start = b > 0 ? hist[b - 1] : 0, end = hist[b];
+    int rank = 0;
+    for (int j = start; j < end; j++) rank += obuf[j] < key;
+    const int pos = start + rank;
+    if (pos < keff) { sv[pos] = v; si[pos] = base_id + (int)(unsigned)key; }
+  }
+  for (int t = keff + tid; t < K; t += BLOCK) { sv[t] = -INFINITY; si[t] = -1; }
+  return true;
+}
+
 template <bool STAGED>
 __global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ logits, long ld,
                                                      const int* __restrict__ row_begin, const int* __restrict__ row_end,
@@ -147,7 +266,7 @@ __global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ l
   int* scratch = hist + HBINS;                     // 16
   float* outv = (float*)(scratch + 16);            // Kp2
   int* outi = (int*)(outv + Kp2);                  // Kp2
-  unsigned* keys = (unsigned*)(outi + Kp2);        // nmax (STAGED only)
+  unsigned* keys = (unsigned*)(outi + Kp2 + 2 * LIN_SPARE);   // nmax (STAGED only); the gap extends the (score, id) buffer
   const int tid = threadIdx.x;
   const long row = blockIdx.x;
   const int cb = max(row_begin ? row_begin[row] : 0, 0);
@@ -161,6 +280,10 @@ __global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ l
 
   auto key_at = [&](int e) -> unsigned { return STAGED ? keys[e] : f2key(src[e]); };
 
+  if (STAGED && sorted && n > 0) {   // single-sweep path, also for rows shorter than K
+    if (linear_select_sort(src, keys, n, K, base_id, hist, scratch, (unsigned long long*)outv, sv, si)) return;
+    __syncthreads();
+  }
   if (n <= K) {
     for (int t = tid; t < Kp2; t += BLOCK) {
       float v = t < n ? src[t] : -INFINITY;
@@ -168,7 +291,7 @@ __global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ l
       outi[t] = (t < n && v > -INFINITY) ? base_id + t : -1;
     }
   } else {
-    if (STAGED) {
+    if (STAGED && !sorted) {
       for (int e = tid; e < n; e += BLOCK) keys[e] = f2key(src[e]);
     }
     // ---- pass 1: bits [31:20] ------------------------------------------------------------
@@ -262,7 +385,7 @@ int dsa_topk_launch(const float* logits, int S, int64_t ld, const int32_t* row_b
   if (S == 0) return DSA_OK;
   int Kp2 = 1;
   while (Kp2 < K) Kp2 <<= 1;
-  const size_t fixed = (size_t)HBINS * 4 + 64 + (size_t)Kp2 * 8;
+  const size_t fixed = (size_t)HBINS * 4 + 64 + (size_t)Kp2 * 8 + (size_t)LIN_SPARE * 8;
   const size_t staged = fixed + (size_t)width * 4;
   const bool use_staged = staged <= 160 * 1024;
   const size_t smem = use_staged ? staged : fixed;
