@@ -348,7 +348,7 @@ Plan layout_plan(int chunk, int Sk, int K) {
   p.W = (chunk + 31) / 32;
   size_t o = 0;
   p.off_bitmap = o; o = align_up(o + (size_t)Sk * p.W * 4);
-  p.off_prefix = o; o = align_up(o + (size_t)Sk * p.W * 4);
+  p.off_prefix = o; o = align_up(o + order::prefix_words(chunk, Sk) * 4);
   p.off_count = o; o = align_up(o + (size_t)(Sk + 1) * 4);
   p.off_start = o; o = align_up(o + (size_t)(Sk + 1) * 4);
   p.off_dst = o; o = align_up(o + (size_t)chunk * K * 4);

@@ -343,9 +343,13 @@ __device__ __forceinline__ void dkv_body(
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
   int* dst_s = ntile_s + 4;
-  for (int t = tid; t < K + BI; t += 256) {
-    const int d = t < K ? dst[(size_t)ql * K + t] : -1;
-    dst_s[t] = d >= 0 ? d : dummy_row;       // invalid slots land in a scratch row: the store count stays fixed
+  for (int t0 = tid; t0 < K + BI; t0 += 8 * 256) {   // eight loads in flight per thread
+    int d[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) d[i] = t0 + i * 256 < K ? dst[(size_t)ql * K + t0 + i * 256] : -1;
+#pragma unroll
+    for (int i = 0; i < 8; i++)       // invalid slots land in a scratch row: the store count stays fixed
+      if (t0 + i * 256 < K + BI) dst_s[t0 + i * 256] = d[i] >= 0 ? d[i] : dummy_row;
   }
   const int ntiles = stage_ids(ids, qi, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
   if (ntiles == 0) return;
@@ -587,7 +591,7 @@ BwdPlan layout_plan(int chunk, int Skv, int K) {
   p.W = (chunk + 31) / 32;
   size_t o = 0;
   p.off_bitmap = o; o = align_up(o + (size_t)Skv * p.W * 4);
-  p.off_prefix = o; o = align_up(o + (size_t)Skv * p.W * 4);
+  p.off_prefix = o; o = align_up(o + order::prefix_words(chunk, Skv) * 4);
   p.off_count = o; o = align_up(o + (size_t)(Skv + 1) * 4);
   p.off_start = o; o = align_up(o + (size_t)(Skv + 1) * 4);
   p.off_dst = o; o = align_up(o + (size_t)chunk * K * 4);

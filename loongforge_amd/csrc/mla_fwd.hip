@@ -84,10 +84,15 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
   int* ntile_s = tlist + NT;
 
   // ---- stage the ids, mark valid slots, list the tiles that have any ---------------------
-  for (int t = tid; t < K; t += 256) {
-    int v = ids[(size_t)qi * K + t];
-    bool ok = (v >= 0) && (v < Skv) && (v <= qpos);
-    idx_s[t] = ok ? v : -1;
+  for (int t0 = tid; t0 < K; t0 += 8 * 256) {     // eight loads in flight per thread
+    int v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = t0 + i * 256 < K ? ids[(size_t)qi * K + t0 + i * 256] : -1;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const bool ok = (v[i] >= 0) && (v[i] < Skv) && (v[i] <= qpos);
+      if (t0 + i * 256 < K) idx_s[t0 + i * 256] = ok ? v[i] : -1;
+    }
   }
   __syncthreads();
   for (int t2 = wave; t2 * 2 < NT; t2 += 4) {

@@ -45,10 +45,15 @@ __device__ __forceinline__ int stage_ids(const int* __restrict__ ids, int qi, in
                                          int* idx_s, unsigned* tmask, int* tlist, int* ntile_s) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int NT = K / BI;
-  for (int t = tid; t < K; t += 256) {
-    int v = ids[(size_t)qi * K + t];
-    bool ok = (v >= 0) && (v < Skv) && (v <= qpos);
-    idx_s[t] = ok ? v : -1;
+  for (int t0 = tid; t0 < K; t0 += 8 * 256) {     // eight loads in flight per thread
+    int v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = t0 + i * 256 < K ? ids[(size_t)qi * K + t0 + i * 256] : -1;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const bool ok = (v[i] >= 0) && (v[i] < Skv) && (v[i] <= qpos);
+      if (t0 + i * 256 < K) idx_s[t0 + i * 256] = ok ? v[i] : -1;
+    }
   }
   __syncthreads();
   for (int t2 = wave; t2 * 2 < NT; t2 += 4) {

@@ -12,15 +12,50 @@ static __global__ void zero_u32_kernel(unsigned* __restrict__ p, size_t n) {
   for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) p[e] = 0u;
 }
 
-// bitmap[key][w] bit b  <=>  local query 32w + b selects key
-static __global__ void bm_set_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv, int q_start,
-                              unsigned* __restrict__ bitmap, int W) {
-  const size_t n = (size_t)cnt * K;
-  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
-    const int ql = (int)(e / K);
-    const int v = ids[(size_t)(q0 + ql) * K + (e % K)];
-    if (v >= 0 && v < Skv && v <= q_start + q0 + ql) atomicOr(&bitmap[(size_t)v * W + (ql >> 5)], 1u << (ql & 31));
+// bitmap[key][w] bit b  <=>  local query 32w + b selects key.
+// Built without global atomics, in two steps.  (1) One workgroup per query sets the query's bits
+// over the keys in LDS and writes them out as one row of qmap[query][key / 32] (Wk words).
+// (2) A transpose of the bit matrix: a wave loads the words of 64 consecutive queries for one key
+// word and turns bit b of all lanes into the 64-bit mask of key 32*kw + b with one ballot; the
+// masks of 4 such query groups are combined through LDS so that every key receives 32 contiguous
+// bytes.
+static __global__ __launch_bounds__(256) void qmap_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv,
+                                                          int q_start, unsigned* __restrict__ qmap, int Wk) {
+  extern __shared__ unsigned qbits[];        // Wk words
+  const int ql = blockIdx.x;
+  for (int w = threadIdx.x; w < Wk; w += 256) qbits[w] = 0u;
+  __syncthreads();
+  for (int t0 = threadIdx.x; t0 < K; t0 += 8 * 256) {
+    int v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = t0 + i * 256 < K ? ids[(size_t)(q0 + ql) * K + t0 + i * 256] : -1;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      if (v[i] >= 0 && v[i] < Skv && v[i] <= q_start + q0 + ql) atomicOr(&qbits[v[i] >> 5], 1u << (v[i] & 31));
   }
+  __syncthreads();
+  for (int w = threadIdx.x; w < Wk; w += 256) qmap[(size_t)ql * Wk + w] = qbits[w];
+}
+
+// grid (ceil(cnt / 256), Wk); workgroup = 4 waves = 256 queries of one key word
+static __global__ __launch_bounds__(256) void bm_transpose_kernel(const unsigned* __restrict__ qmap, int cnt, int Skv, int Wk,
+                                                                  unsigned* __restrict__ bitmap, int W) {
+  __shared__ unsigned long long mask_s[32][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kw = blockIdx.y;
+  const int ql = blockIdx.x * 256 + threadIdx.x;
+  const unsigned word = ql < cnt ? qmap[(size_t)ql * Wk + kw] : 0u;
+#pragma unroll
+  for (int b = 0; b < 32; b++) {
+    const unsigned long long m = __ballot((word >> b) & 1u);
+    if (lane == b) mask_s[b][wave] = m;
+  }
+  __syncthreads();
+  // thread t < 256: key bit t / 8, 32-bit piece t % 8 of the 256 queries of this workgroup
+  const int b = threadIdx.x >> 3, piece = threadIdx.x & 7;
+  const int key = kw * 32 + b;
+  const int w = blockIdx.x * 8 + piece;
+  if (key < Skv && w < W) bitmap[(size_t)key * W + w] = ((const unsigned*)&mask_s[b][0])[piece];
 }
 
 // prefix[key][w] = number of set bits in words < w; count[key] = total.  One wave per key.
@@ -87,10 +122,21 @@ static __global__ void rank_kernel(const int* __restrict__ ids, int q0, int cnt,
 
 // Launches the five kernels above for queries [q0, q0 + cnt).  A slot counts when its id v is in
 // [0, Skv) and v <= q_start + (query index); pass a huge q_start to accept every id in range.
+// The prefix buffer doubles as the scratch of step (1) (cnt * ceil(Skv / 32) words; it is rewritten by
+// the prefix pass afterwards): size it with prefix_words().
+inline size_t prefix_words(int chunk, int Skv) {
+  const size_t W = (size_t)(chunk + 31) / 32, Wk = (size_t)(Skv + 31) / 32;
+  return (size_t)Skv * W > (size_t)chunk * Wk ? (size_t)Skv * W : (size_t)chunk * Wk;
+}
 inline void build(const int* ids, int q0, int cnt, int K, int Skv, int q_start, unsigned* bitmap, unsigned* prefix,
                   int* count, int* start, int* dst, int W, hipStream_t st) {
-  zero_u32_kernel<<<dim3(1024), dim3(256), 0, st>>>(bitmap, (size_t)Skv * W);
-  bm_set_kernel<<<dim3(2048), dim3(256), 0, st>>>(ids, q0, cnt, K, Skv, q_start, bitmap, W);
+  const int Wk = (Skv + 31) / 32;
+  unsigned* qmap = prefix;
+  if ((size_t)Wk * 4 > 48 * 1024)
+    (void)hipFuncSetAttribute((const void*)qmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Wk * 4);
+  qmap_kernel<<<dim3(cnt), dim3(256), (size_t)Wk * 4, st>>>(ids, q0, cnt, K, Skv, q_start, qmap, Wk);
+  // every word of the bitmap is written (zeros beyond the last query), so no clearing pass is needed
+  bm_transpose_kernel<<<dim3((W + 7) / 8, Wk), dim3(256), 0, st>>>(qmap, cnt, Skv, Wk, bitmap, W);
   bm_prefix_kernel<<<dim3((Skv + 3) / 4), dim3(256), 0, st>>>(bitmap, prefix, count, Skv, W);
   key_scan_kernel<<<dim3(1), dim3(1024), 0, st>>>(count, start, Skv);
   rank_kernel<<<dim3(2048), dim3(256), 0, st>>>(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, start, W, dst);
