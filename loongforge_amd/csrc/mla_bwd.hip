@@ -189,8 +189,12 @@ __global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
 // ---------------------------------------------------------------------------------------------
 // dQ^T[d, head] += KV^T[d, key] . dS^T[key, head] per 32-key tile.  Both operands are LDS transpose
 // reads: of the gathered key tile (18 d-tiles) and of the tile's dS block copied verbatim from the
-// pass-A buffer.  The 18 accumulator tiles of a wave (288 registers) sit in the 256 accumulation
-// registers plus 32 architectural ones.
+// pass-A buffer.  The 72 accumulator tiles (18 d-tiles x 4 head groups) are split over the waves
+// by d: wave w owns d-tiles 4w .. 4w+3 for all four head groups, plus d-tile 16 + w/2 for head
+// groups 2(w%2), 2(w%2)+1 - 18 tiles (288 registers: 256 accumulation + 32 architectural) and 36
+// MFMAs per wave and tile.  A key-tile operand read from LDS then feeds up to four MFMAs, and the
+// eight dS operands of a tile are read once per wave: 72 KB of LDS reads per tile instead of the
+// 152 KB of a split by heads.
 template <int STAGES>
 __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
     const __bf16* __restrict__ kv, const int* __restrict__ ids, const unsigned char* __restrict__ pds,
@@ -210,8 +214,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
 
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
   const LaneOffsets lo = lane_offsets();
-  // transposed read of the dS block [wave][s'][g'][key][8 heads]: lane (blk, ii) points at key
-  // 16s + 8t + 4g + ii/4 and the 4 heads 16*(blk&1) + 4*(ii&3) .. +3 of this wave
+  // transposed read of the dS block [head group][s'][g'][key][8 heads]: lane (blk, ii) points at
+  // key 16s + 8t + 4g + ii/4 and the 4 heads 16*(blk&1) + 4*(ii&3) .. +3 of a head group
   unsigned ds_off[2][2];
   {
     const int blk = lane >> 4, ii = lane & 15, qq = ii & 3;
@@ -220,9 +224,27 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         const int key = 16 * s + 8 * t + 4 * g + (ii >> 2);
-        ds_off[s][t] = (unsigned)(TILE_BYTES + wave * 2048 + (blk & 1) * 1024 + (qq & 1) * 512 + key * 16 + (qq >> 1) * 8);
+        ds_off[s][t] = (unsigned)(TILE_BYTES + (blk & 1) * 1024 + (qq & 1) * 512 + key * 16 + (qq >> 1) * 8);
       }
   }
+  // key-tile operand offsets of this wave's d-tiles: i = 0..3 -> d-tile 4*wave + i, i = 4 -> 16 + wave/2
+  const unsigned grp_main = (unsigned)(2 * wave) * GRP_BYTES;          // (4w + i) >> 1 = 2w + (i >> 1)
+  const unsigned grp_last = (unsigned)(8 * GRP_BYTES);                 // (16 + w/2) >> 1 = 8
+  const int par_last = (wave >> 1) & 1;
+  unsigned tr_last[2][2];
+  {
+    // same formula as LaneOffsets::tr_off, with the parity of the d-tile known only at run time
+    const int blk = lane >> 4, ii = lane & 15;
+    const int cl = 2 * (blk & 1) + ((ii & 3) >> 1), half = ii & 1;
+#pragma unroll
+    for (int s = 0; s < 2; s++)
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const int key = 16 * s + 8 * t + 4 * g + (ii >> 2);
+        tr_last[s][t] = (unsigned)(key * 128 + (((4 * par_last + cl) ^ swz(key)) << 4) + half * 8) + grp_last;
+      }
+  }
+  const int hg_last = 2 * (wave & 1);
   auto issue = [&](int n) {
     const int tile = tlist[n];
     const unsigned sb = lds0 + (unsigned)((n % STAGES) * STAGE_BYTES);
@@ -233,64 +255,81 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
     dma16(lb + 4096, (unsigned)(4096 + tid * 16), src);
   };
 
-  f32x16 acc[18];
+  f32x16 acc[18];     // u < 16: d-tile 4*wave + u/4, head group u%4; u = 16, 17: d-tile 16 + wave/2, head group hg_last + u - 16
 #pragma unroll
-  for (int dt = 0; dt < 18; dt++) {
+  for (int u = 0; u < 18; u++) {
 #pragma unroll
-    for (int e = 0; e < 16; e++) acc[dt][e] = 0.f;
-    if (dt < 16) asm volatile("" : "+a"(acc[dt])); else asm volatile("" : "+v"(acc[dt]));
+    for (int e = 0; e < 16; e++) acc[u][e] = 0.f;
+    if (u < 16) asm volatile("" : "+a"(acc[u])); else asm volatile("" : "+v"(acc[u]));
   }
+  typedef short i16x8 __attribute__((ext_vector_type(8)));
+  auto tr_pair = [&](const unsigned char* p0, const unsigned char* p1) {
+    const i16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, p0));
+    const i16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, p1));
+    return __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
   for (int n = 0; n < STAGES - 1 && n < ntiles; n++) issue(n);
   for (int n = 0; n < ntiles; n++) {
     wait_vmcnt_le(11 * min(STAGES - 2, ntiles - 1 - n));
     __syncthreads();
     if (n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
     const unsigned char* tb = smem + (n % STAGES) * STAGE_BYTES;
-    typedef short i16x8 __attribute__((ext_vector_type(8)));
-    bf16x8 bds[2];
+    // the eight dS operands of the tile: [head group][k-step]
+    bf16x8 bds[4][2];
 #pragma unroll
-    for (int s = 0; s < 2; s++) {
-      i16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, tb + ds_off[s][0]));
-      i16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, tb + ds_off[s][1]));
-      bds[s] = __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
-    }
-    i16x4 v[2][2][2];
+    for (int hg = 0; hg < 4; hg++)
 #pragma unroll
-    for (int dt = 0; dt < 2; dt++)
+      for (int s = 0; s < 2; s++) bds[hg][s] = tr_pair(tb + hg * 2048 + ds_off[s][0], tb + hg * 2048 + ds_off[s][1]);
+    // key-tile operands, one d-tile ahead
+    bf16x8 a[2][2];
 #pragma unroll
-      for (int s = 0; s < 2; s++)
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-          v[dt][s][t] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, tb + (dt >> 1) * GRP_BYTES + lo.tr_off[s][t][dt & 1]));
+    for (int s = 0; s < 2; s++)
+      a[0][s] = tr_pair(tb + grp_main + lo.tr_off[s][0][0], tb + grp_main + lo.tr_off[s][1][0]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int dt = 0; dt < 18; dt++) {
+    for (int i = 0; i < 5; i++) {
+      if (i + 1 < 5) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          if (i + 1 < 4)
+            a[(i + 1) & 1][s] = tr_pair(tb + grp_main + ((i + 1) >> 1) * GRP_BYTES + lo.tr_off[s][0][(i + 1) & 1],
+                                        tb + grp_main + ((i + 1) >> 1) * GRP_BYTES + lo.tr_off[s][1][(i + 1) & 1]);
+          else
+            a[(i + 1) & 1][s] = tr_pair(tb + tr_last[s][0], tb + tr_last[s][1]);
+        }
+      }
 #pragma unroll
       for (int s = 0; s < 2; s++) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(v[dt & 1][s][0], v[dt & 1][s][1], 0, 1, 2, 3, 4, 5, 6, 7));
-        if (dt < 16) mfma_a_vv(acc[dt], a, bds[s]);
-        else mfma_v_vv(acc[dt], a, bds[s]);
-      }
-      if (dt + 2 < 18) {
+        if (i < 4) {
 #pragma unroll
-        for (int s = 0; s < 2; s++)
-#pragma unroll
-          for (int t = 0; t < 2; t++)
-            v[dt & 1][s][t] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, tb + ((dt + 2) >> 1) * GRP_BYTES + lo.tr_off[s][t][dt & 1]));
+          for (int hg = 0; hg < 4; hg++) mfma_a_vv(acc[4 * i + hg], a[i & 1][s], bds[hg][s]);
+        } else {
+          // head groups hg_last, hg_last + 1 (a branch, so that no register array is indexed at run time)
+          if (hg_last) {
+            mfma_v_vv(acc[16], a[i & 1][s], bds[2][s]);
+            mfma_v_vv(acc[17], a[i & 1][s], bds[3][s]);
+          } else {
+            mfma_v_vv(acc[16], a[i & 1][s], bds[0][s]);
+            mfma_v_vv(acc[17], a[i & 1][s], bds[1][s]);
+          }
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  const int h = wave * 32 + r;
-  if (h < H) {
-    unsigned short* op = (unsigned short*)dq + ((size_t)qi * H + h) * DQK + 4 * g;
+  // ---- write dQ: accumulator e of a lane is d = 32*dt + 8*(e/4) + 4*g + (e%4), head = 32*hg + r ----
 #pragma unroll
-    for (int dt = 0; dt < 18; dt++) {
-      if (dt < 16) mfma_done_a(acc[dt]); else mfma_done_v(acc[dt]);
+  for (int u = 0; u < 18; u++) {
+    if (u < 16) mfma_done_a(acc[u]); else mfma_done_v(acc[u]);
+    const int dt = u < 16 ? 4 * wave + (u >> 2) : 16 + (wave >> 1);
+    const int hg = u < 16 ? (u & 3) : hg_last + (u - 16);
+    const int h = hg * 32 + r;
+    if (h < H) {
+      unsigned short* op = (unsigned short*)dq + ((size_t)qi * H + h) * DQK + 32 * dt + 4 * g;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        uint2 w = make_uint2(pack_bf16x2(acc[dt][4 * j], acc[dt][4 * j + 1]), pack_bf16x2(acc[dt][4 * j + 2], acc[dt][4 * j + 3]));
-        *(uint2*)(op + 32 * dt + 8 * j) = w;
+        uint2 w = make_uint2(pack_bf16x2(acc[u][4 * j], acc[u][4 * j + 1]), pack_bf16x2(acc[u][4 * j + 2], acc[u][4 * j + 3]));
+        *(uint2*)(op + 8 * j) = w;
       }
     }
   }
