@@ -26,9 +26,11 @@ constexpr int KSTEPS = DQK / 16;             // 36
 constexpr int DTILES = DV / 32;              // 16
 constexpr float LOG2E = 1.4426950408889634f;
 
-// 16-byte slot swizzle of key row r inside its 128-byte group: any 8 consecutive rows hit 8
-// different slots and rows r, r+8 differ as well.
-__device__ __forceinline__ int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+// 16-byte slot swizzle of key row r inside its 128-byte group: conflict-free for the 128-bit row
+// reads (16 lanes) and for the transpose reads (32 lanes) of this kernel.
+__device__ __forceinline__ int swz(int r) {
+  return (((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1) | ((r ^ (r >> 3)) & 1);
+}
 
 __device__ __forceinline__ void dma16(unsigned lds_base, unsigned goff, const void* gbase) {
   // Each lane fetches 16 bytes at gbase + goff; the wave's 64 chunks land at lds_base + 16*lane.

@@ -15,10 +15,14 @@ constexpr int VSTEPS = DV / 16;              // 32 MFMA k-steps over d_v
 constexpr float LOG2E = 1.4426950408889634f;
 
 // A key row (1152 bytes) is stored as nine 128-byte groups; group p of all 32 rows is contiguous
-// (GRP_BYTES).  Inside a group the 16-byte slot of chunk c of row r is (c & 7) ^ swz(r): any 8
-// consecutive rows hit 8 different slots and rows r, r+8 differ as well, so 128-bit row reads by
-// 32 lanes and transpose reads by 16 lanes are spread over the banks.
-__device__ __forceinline__ int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+// (GRP_BYTES).  Inside a group the 16-byte slot of chunk c of row r is (c & 7) ^ swz(r).  swz
+// permutes the bits of r so that (a) the rows of one parity in any aligned block of 16 hit 8
+// different slots - 128-bit row reads by 16 lanes are conflict free - and (b) bit 2 of the slot
+// follows bit 1 of the row, so the four keys a transpose read touches in a half wave fall into
+// four different 64-byte bank regions - transpose reads by 32 lanes are conflict free as well.
+__device__ __forceinline__ int swz(int r) {
+  return (((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1) | ((r ^ (r >> 3)) & 1);
+}
 
 // Each lane fetches 16 bytes at gbase + goff; the wave's 64 chunks land at lds_base + 16*lane.
 // (m0 carries the LDS base; nothing else in these kernels uses m0.)  The transfer is counted by
