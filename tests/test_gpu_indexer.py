@@ -142,3 +142,47 @@ def test_relative_layout_of_packed_logits(gpu):
         n = int(ke[i] - ks[i])
         assert torch.equal(rel[i, :n], dense[i, int(ks[i]): int(ke[i])])
         assert torch.isinf(rel[i, n:]).all()
+
+
+@pytest.mark.parametrize("kind", ["normal", "ties", "constant", "outlier", "holes", "short", "two_values"])
+@pytest.mark.parametrize("K,sorted_out", [(2048, True), (1000, True), (256, True), (512, False)])
+def test_topk_rule_on_crafted_rows(gpu, kind, K, sorted_out):
+    """The selection rule on rows that exercise every branch of the kernel: the K largest values, ties
+    broken towards the smaller column, output in descending score / ascending column order.  The
+    expectation is a stable sort by the library routine."""
+    from loongforge_amd import ops
+
+    n, rows = 6000, 12
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(rows, n, generator=g)
+    if kind == "ties":
+        x = torch.round(x * 8) / 8                        # a few dozen distinct values
+    elif kind == "constant":
+        x = torch.full((rows, n), 1.25)
+    elif kind == "outlier":
+        x[:, 17] = 1e30                                   # every other value lands in the last value bins
+        x[:, 99] = -1e30
+    elif kind == "holes":
+        x[torch.rand(rows, n, generator=g) < 0.3] = float("-inf")
+    elif kind == "two_values":
+        x = (x > 0.5).float()
+    end = torch.full((rows,), n, dtype=torch.int32)
+    if kind == "short":
+        end = torch.tensor([1, 2, 63, 64, 255, 256, 257, 999, 1000, 1001, 2047, 2049], dtype=torch.int32)
+    beg = torch.zeros(rows, dtype=torch.int32)
+    sc, ids = ops.topk(x.to(gpu), K, beg.to(gpu), end.to(gpu), sorted=sorted_out)
+    sc, ids = sc.cpu(), ids.cpu()
+    for i in range(rows):
+        row = x[i, : int(end[i])]
+        order = torch.sort(-row, stable=True).indices      # descending value, ascending column among equals
+        fin = torch.isfinite(row[order])
+        exp_ids = order[fin][:K]
+        kk = len(exp_ids)
+        if sorted_out:
+            assert torch.equal(ids[i, :kk].long(), exp_ids), (kind, K, i)
+            assert torch.equal(sc[i, :kk], row[exp_ids])
+        else:
+            got = ids[i][ids[i] >= 0].long()
+            assert torch.equal(torch.sort(got).values, torch.sort(exp_ids).values), (kind, K, i)
+            assert torch.equal(sc[i][ids[i] >= 0], row[got])
+        assert (ids[i, kk:] == -1).all() and torch.isinf(sc[i, kk:]).all() and (sc[i, kk:] < 0).all()
