@@ -23,10 +23,13 @@ constexpr int D = 128;
 constexpr int TK = 128;                 // slots per tile
 constexpr int TILE_BYTES = TK * D;      // fp8 key rows
 constexpr int RED_STRIDE = 132;         // floats per head row of the cross-wave reduction buffer
+constexpr int STRIP_STRIDE = 144;       // bytes per key row of the d_k transpose strip (128 + bank spread)
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+__device__ __forceinline__ int kb_swz(int key) { return ((key & 3) << 2) | ((key >> 2) & 3); }
+__device__ __forceinline__ int es_swz(int key) { return 2 * ((key >> 1) & 3) + ((key >> 3) & 1); }
 __device__ __forceinline__ void dma16(unsigned lds_base, unsigned goff, const void* gbase) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :: "s"(lds_base), "v"(goff), "s"(gbase) : "memory");
@@ -58,26 +61,42 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int HI = 32 * NHT;
   // [2][TILE_BYTES] fp8 key tiles | kb [4 waves][32 keys][256 B] bf16 keys | es [4 waves][2][32 keys][HI] bf16 E |
-  // idx_s [K] | a_s [K] | dst_s [K] | dw_red [4][64]
+  // idx_s [K] | a_s [K] | dst_s [K] | dw_red [4][64] | strip [4 waves][32][STRIP_STRIDE]
   unsigned char* kb = smem + 2 * TILE_BYTES;
   unsigned char* es = kb + 4 * 32 * 256;
   int* idx_s = (int*)(es + 4 * 2 * 32 * 128);
   float* a_s = (float*)(idx_s + K);
   int* dst_s = (int*)(a_s + K);
   float* dw_red = (float*)(dst_s + K);
+  unsigned char* strip = (unsigned char*)(dw_red + 4 * 64) + (threadIdx.x >> 6) * (32 * STRIP_STRIDE);   // per wave
   float* red = (float*)smem;                        // [HI][RED_STRIDE], reuses the tile area at the end
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, g = lane >> 5;
   const int ql = cnt - 1 - (int)blockIdx.x;
   const int qi = q0 + ql;
 
-  for (int t = tid; t < K; t += 256) {
-    const int v = ids[(size_t)qi * K + t];
-    const bool ok = v >= 0 && v < Sk;
-    idx_s[t] = ok ? v : -1;
-    a_s[t] = ok ? gsc[(size_t)qi * K + t] * k_scale[v] : 0.f;
-    const int d = dst[(size_t)ql * K + t];
-    dst_s[t] = (ok && d >= 0) ? d : dummy_row;
+  for (int t0 = tid; t0 < K; t0 += 8 * 256) {     // eight slots per thread with all their loads in flight
+    int v[8], d[8];
+    float gv[8], kv[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int t = min(t0 + i * 256, K - 1);
+      v[i] = ids[(size_t)qi * K + t];
+      gv[i] = gsc[(size_t)qi * K + t];
+      d[i] = dst[(size_t)ql * K + t];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) kv[i] = k_scale[(v[i] >= 0 && v[i] < Sk) ? v[i] : 0];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int t = t0 + i * 256;
+      if (t < K) {
+        const bool ok = v[i] >= 0 && v[i] < Sk;
+        idx_s[t] = ok ? v[i] : -1;
+        a_s[t] = ok ? gv[i] * kv[i] : 0.f;
+        dst_s[t] = (ok && d[i] >= 0) ? d[i] : dummy_row;
+      }
+    }
   }
   // stage q8[i] (HI x 128 bytes) in the kb area to build the transposed bf16 operand
   for (int c = tid; c < HI * 8; c += 256) *(uint4*)(kb + c * 16) = *(const uint4*)(q8 + (size_t)qi * HI * D + c * 16);
@@ -137,14 +156,22 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
     for (int x = 0; x < 2; x++) b_off[s][x] = (unsigned)((32 * wave + r) * D + (((4 * s + 2 * g + x) ^ swz(r)) << 4));
   const int blk = lane >> 4, ii = lane & 15;
   // transpose reads: lane (blk, ii) points at key 16*s2 + 8*t + 4*g + ii/4, column chunk 16*(blk&1) + 4*(ii&3)
-  unsigned kt_off[2][2], et_off[2][2];
+  // Both wave-private buffers XOR the 16-byte slot index with a permutation of the key's bits
+  // (kb_swz: 16 slots per 256-byte row, es_swz: 8 slots per 128-byte row), chosen so that the
+  // row-wise writes by 16 lanes and the transpose reads by 32 lanes spread over all banks.
+  unsigned kt_off[2][2][4], et_off[2][2][NHT];
 #pragma unroll
   for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
     for (int t = 0; t < 2; t++) {
       const int key = 16 * s2 + 8 * t + 4 * g + (ii >> 2);
-      kt_off[s2][t] = (unsigned)(wave * 8192 + key * 256 + (16 * (blk & 1) + 4 * (ii & 3)) * 2);
-      et_off[s2][t] = (unsigned)(wave * 8192 + key * 128 + (16 * (blk & 1) + 4 * (ii & 3)) * 2);
+      const int sub = 2 * (blk & 1) + ((ii & 3) >> 1), half = (ii & 1) * 8;
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++)
+        kt_off[s2][t][dt] = (unsigned)(wave * 8192 + key * 256 + (((4 * dt + sub) ^ kb_swz(key)) << 4) + half);
+#pragma unroll
+      for (int tt = 0; tt < NHT; tt++)
+        et_off[s2][t][tt] = (unsigned)(wave * 8192 + key * 128 + (((4 * tt + sub) ^ es_swz(key)) << 4) + half);
     }
 
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
@@ -189,7 +216,7 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
 #pragma unroll
       for (int e = 0; e < 16; e++) {
         const float rr = acc[e];
-        dwp[tt][e] = fmaf(a, fmaxf(rr, 0.f), dwp[tt][e]);
+        dwp[tt][e] = fmaf(a, __builtin_bit_cast(float, max(__builtin_bit_cast(int, rr), 0)), dwp[tt][e]);   // relu on the bit pattern
         const float ev = rr > 0.f ? a * wq[tt][e] : 0.f;
         const __bf16 h = (__bf16)ev;
         ehi[tt][e >> 3][e & 7] = h;
@@ -200,10 +227,16 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
 
     // ---- d_k8 rows: row^T[d, key] = Q^T . E, 32 keys of this wave --------------------------------
     {
-      float* rowp = rows + (size_t)dst_s[slot] * D + 4 * g;
+      // The 32 x 32 fp32 block of a d-tile is transposed through a wave-private LDS strip, so that a
+      // store instruction writes eight complete 128-byte row segments (lane: key 8*i + lane/8,
+      // 16-byte piece lane%8) instead of 32 scattered 32-byte pieces.
+      float* rowp[4];
 #pragma unroll
-      for (int dt = 0; dt < 4; dt++) {
-        f32x16 racc;
+      for (int i = 0; i < 4; i++)
+        rowp[i] = rows + (size_t)dst_s[t * TK + 32 * wave + 8 * i + (lane >> 3)] * D + 4 * (lane & 7);
+      unsigned char* sw = strip + r * STRIP_STRIDE + 16 * g;
+      const unsigned char* sr = strip + (lane >> 3) * STRIP_STRIDE + (lane & 7) * 16;
+      auto row_mfmas = [&](int dt, f32x16& racc) {
         mfma_v_av_first(racc, qt[dt][0], ehi[0][0]);
         mfma_v_av(racc, qt[dt][0], elo[0][0]);
 #pragma unroll
@@ -211,12 +244,23 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
           mfma_v_av(racc, qt[dt][kk], ehi[kk >> 1][kk & 1]);
           mfma_v_av(racc, qt[dt][kk], elo[kk >> 1][kk & 1]);
         }
-        mfma_done_v(racc);
+      };
+      f32x16 racc[2];
+      row_mfmas(0, racc[0]);
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++) {
+        // the next d-tile's MFMAs run while this one goes through the strip and out to memory
+        if (dt + 1 < 4) row_mfmas(dt + 1, racc[(dt + 1) & 1]);
+        else mfma_done_v(racc[dt & 1]);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-          const f32x4 w = {racc[4 * j], racc[4 * j + 1], racc[4 * j + 2], racc[4 * j + 3]};
-          *(f32x4*)(rowp + 32 * dt + 8 * j) = w;
+          const f32x4 w = {racc[dt & 1][4 * j], racc[dt & 1][4 * j + 1], racc[dt & 1][4 * j + 2], racc[dt & 1][4 * j + 3]};
+          *(f32x4*)(sw + 32 * j) = w;                // d = 32*dt + 8*j + 4*g .. +3 of key r
         }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 4; i++) *(f32x4*)(rowp[i] + 32 * dt) = *(const f32x4*)(sr + 8 * i * STRIP_STRIDE);
+        __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -225,7 +269,8 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
     {
       // lane (key r, half g) converts bytes [64g, 64g + 64) of its key row
       const unsigned char* krow = tb + (32 * wave + r) * D;
-      unsigned char* kdst = kb + wave * 8192 + r * 256 + g * 128;
+      unsigned char* kdst = kb + wave * 8192 + r * 256;
+      const int ksw = kb_swz(r);
 #pragma unroll
       for (int c = 0; c < 4; c++) {
         const int slot16 = (4 * g + c) ^ swz(r);
@@ -241,16 +286,17 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
                                                                : __builtin_amdgcn_cvt_f32_fp8(w[x], 3));
             if (x < 2) o0[4 * x + y] = v; else o1[4 * (x - 2) + y] = v;
           }
-        *(bf16x8*)(kdst + c * 32) = o0;
-        *(bf16x8*)(kdst + c * 32 + 16) = o1;
+        *(bf16x8*)(kdst + (((8 * g + 2 * c) ^ ksw) << 4)) = o0;
+        *(bf16x8*)(kdst + (((8 * g + 2 * c + 1) ^ ksw) << 4)) = o1;
       }
       // E[key r][heads]: the lane holds heads 32*tt + 8*j + 4*g + (0..3)
       unsigned char* edst = es + wave * 8192 + r * 128;
+      const int esw = es_swz(r);
 #pragma unroll
       for (int tt = 0; tt < NHT; tt++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-          const int hb = (32 * tt + 8 * j + 4 * g) * 2;
+          const int hb = (((4 * tt + j) ^ esw) << 4) + 8 * g;      // heads 32*tt + 8*j + 4*g .. +3
           bf16x4 vh, vl;
 #pragma unroll
           for (int e = 0; e < 4; e++) { vh[e] = ehi[tt][j >> 1][4 * (j & 1) + e]; vl[e] = elo[tt][j >> 1][4 * (j & 1) + e]; }
@@ -263,12 +309,12 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
         bf16x8 bh[NHT], bl[NHT];
 #pragma unroll
         for (int tt = 0; tt < NHT; tt++) {
-          bh[tt] = tr_pair(es + et_off[s2][0] + 64 * tt, es + et_off[s2][1] + 64 * tt);
-          bl[tt] = tr_pair(es + 4096 + et_off[s2][0] + 64 * tt, es + 4096 + et_off[s2][1] + 64 * tt);
+          bh[tt] = tr_pair(es + et_off[s2][0][tt], es + et_off[s2][1][tt]);
+          bl[tt] = tr_pair(es + 4096 + et_off[s2][0][tt], es + 4096 + et_off[s2][1][tt]);
         }
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) {
-          const bf16x8 ak = tr_pair(kb + kt_off[s2][0] + 64 * dt, kb + kt_off[s2][1] + 64 * dt);
+          const bf16x8 ak = tr_pair(kb + kt_off[s2][0][dt], kb + kt_off[s2][1][dt]);
 #pragma unroll
           for (int tt = 0; tt < NHT; tt++) {
             mfma_a_vv(dq_acc[tt][dt], ak, bh[tt]);
@@ -397,7 +443,7 @@ extern "C" int dsa_indexer_bwd(const float* g, const void* q8, const void* k8, c
   int* start = (int*)(ws + p.off_start);
   int* dstp = (int*)(ws + p.off_dst);
   float* rows = (float*)(ws + p.off_rows);
-  size_t smem = (size_t)2 * TILE_BYTES + 4 * 32 * 256 + 4 * 2 * 32 * 128 + (size_t)K * 12 + 4 * 64 * 4;
+  size_t smem = (size_t)2 * TILE_BYTES + 4 * 32 * 256 + 4 * 2 * 32 * 128 + (size_t)K * 12 + 4 * 64 * 4 + 4 * 32 * STRIP_STRIDE;
   const size_t red_bytes = (size_t)Hi * RED_STRIDE * 4;
   if (red_bytes > (size_t)2 * TILE_BYTES + 4 * 32 * 256) smem += red_bytes;
   auto kern = Hi == 32 ? indexer_bwd_kernel<1> : indexer_bwd_kernel<2>;
