@@ -40,6 +40,19 @@ int dsa_quant_rowwise_e4m3(const void* x, int64_t rows, int cols, void* x8, floa
                            float eps, int pow2, void* stream);
 
 /*
+ * Hadamard rotation fused with the quantiser above: y = bf16(H_128 . x * 128^-0.5) (Sylvester
+ * order), then (x8, scale_inv) = quantise(y).  Replaces the pair rotate_activation ->
+ * Float8BlockQuantizer of the indexer front end: rotate_activation at
+ * loongforge/models/common/experimental_attention_variant/dsa_fused.py:74-90 (applied at :604-606)
+ * followed by the quantiser at dsa_fused_kernels.py:2341-2346, without the bf16 round trip
+ * through memory.  Either output may be NULL: x8 == NULL gives the rotation only (y), y == NULL the
+ * quantised payload only.
+ *   x, y [rows, 128] bf16     x8 [rows, 128] fp8-e4m3 (OCP)     scale_inv [rows] f32
+ */
+int dsa_rotate_quant_e4m3(const void* x, int64_t rows, int cols, void* x8, float* scale_inv, void* y,
+                          float eps, int pow2, void* stream);
+
+/*
  * Lightning-indexer logits:
  *   logits[i, j - base_i] = k_scale[j] * sum_h q_w[i,h] * relu(q8[i,h,:] . k8[j,:]),  ks[i] <= j < ke[i]
  * and -inf for every other column of row i.  base_i = 0 when `relative` == 0 (dense layout, width

@@ -49,7 +49,86 @@ __global__ __launch_bounds__(256) void quant128_kernel(const uint4* __restrict__
   }
 }
 
+// Hadamard rotation of a 128-element row (Sylvester order, scaled by 128^-0.5, rounded to bf16 as the
+// unfused sequence "fp32 product with the Hadamard matrix -> bf16" does) followed by the same
+// quantiser.  The butterfly runs over the 7 index bits: 3 inside a lane's 8 elements, 4 across the
+// 16 lanes of a row.  Either output may be absent (x8 == nullptr: rotation only; y == nullptr:
+// quantised payload only).
+__global__ __launch_bounds__(256) void rotate_quant128_kernel(const uint4* __restrict__ x, uint2* __restrict__ x8,
+                                                              float* __restrict__ scale_inv, uint4* __restrict__ y,
+                                                              int64_t rows, float eps, int pow2) {
+  int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  int sub = threadIdx.x & 15;
+  bool live = row < rows;
+  uint4 raw = live ? x[row * 16 + sub] : make_uint4(0, 0, 0, 0);
+  unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+    v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+  }
+#pragma unroll
+  for (int m = 1; m < 8; m <<= 1)
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      if (!(i & m)) { const float a = v[i], b = v[i | m]; v[i] = a + b; v[i | m] = a - b; }
+#pragma unroll
+  for (int m = 1; m < 16; m <<= 1)
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const float o = __shfl_xor(v[i], m, 64);
+      v[i] = (sub & m) ? o - v[i] : v[i] + o;
+    }
+  unsigned yb[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const unsigned lo = f32_to_bf16_bits(v[2 * i] * 0.08838834764831845f), hi = f32_to_bf16_bits(v[2 * i + 1] * 0.08838834764831845f);
+    yb[i] = lo | (hi << 16);
+    v[2 * i] = __builtin_bit_cast(float, lo << 16);
+    v[2 * i + 1] = __builtin_bit_cast(float, hi << 16);
+  }
+  if (live && y) y[row * 16 + sub] = make_uint4(yb[0], yb[1], yb[2], yb[3]);
+  if (!x8) return;
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(v[i]));
+  amax = wave_max16(amax);
+  amax = fmaxf(amax, eps);
+  float scale = 448.0f / amax;
+  if (pow2) scale = __builtin_bit_cast(float, __builtin_bit_cast(unsigned, scale) & 0xff800000u);
+  float q[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) q[i] = fminf(fmaxf(v[i] * scale, -448.0f), 448.0f);
+  int lo = 0, hi = 0;
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], lo, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], lo, true);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], hi, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], hi, true);
+  if (live) {
+    x8[row * 16 + sub] = make_uint2((unsigned)lo, (unsigned)hi);
+    if (sub == 0) scale_inv[row] = 1.0f / scale;
+  }
+}
+
 }  // namespace
+
+extern "C" int dsa_rotate_quant_e4m3(const void* x, int64_t rows, int cols, void* x8, float* scale_inv, void* y,
+                                     float eps, int pow2, void* stream) {
+  DSA_REQUIRE(cols == 128, "dsa_rotate_quant_e4m3: only rows of 128 elements are supported, got %d", cols);
+  DSA_REQUIRE(rows >= 0, "dsa_rotate_quant_e4m3: negative row count");
+  DSA_REQUIRE(x8 != nullptr || y != nullptr, "dsa_rotate_quant_e4m3: no output requested");
+  DSA_REQUIRE(x8 == nullptr || scale_inv != nullptr, "dsa_rotate_quant_e4m3: payload without scales");
+  DSA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)x8 % 8) == 0 && ((uintptr_t)y % 16) == 0,
+              "dsa_rotate_quant_e4m3: misaligned pointer");
+  if (rows == 0) return DSA_OK;
+  int64_t blocks = (rows + 15) / 16;
+  DSA_REQUIRE(blocks < (1ll << 31), "dsa_rotate_quant_e4m3: too many rows");
+  rotate_quant128_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+      (const uint4*)x, (uint2*)x8, scale_inv, (uint4*)y, rows, eps, pow2);
+  DSA_CHECK_LAUNCH("dsa_rotate_quant_e4m3");
+  return DSA_OK;
+}
 
 extern "C" int dsa_quant_rowwise_e4m3(const void* x, int64_t rows, int cols, void* x8, float* scale_inv,
                                       float eps, int pow2, void* stream) {

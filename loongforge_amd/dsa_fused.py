@@ -163,8 +163,10 @@ class DSAIndexerFused(MegatronModule):
                                     mscale=mscale, cp_group=self.pg_collection.cp)
         return torch.cat([x_pe, x_nope], dim=-1)
 
-    def get_query_key_weight_tensors(self, x, qr, packed_seq_params: Optional[PackedSeqParams] = None):
-        """q ``[s, (b,) h, d]``, k ``[s, (b,) d]``, weights ``[s, (b,) h]`` (dsa_fused.py:490-638)."""
+    def get_query_key_weight_tensors(self, x, qr, packed_seq_params: Optional[PackedSeqParams] = None,
+                                     defer_rotation: bool = False):
+        """q ``[s, (b,) h, d]``, k ``[s, (b,) d]``, weights ``[s, (b,) h]`` (dsa_fused.py:490-638).
+        ``defer_rotation`` leaves the Hadamard rotation to the caller (the indexer kernel fuses it)."""
         x = x.detach()
         qr = qr.detach()
         rotary_seq_len = self.rotary_pos_emb.get_rotary_seq_len(None, None, x, self.config, packed_seq_params)
@@ -194,7 +196,7 @@ class DSAIndexerFused(MegatronModule):
         else:
             k = self._apply_rope(k.unsqueeze(-2), rotary_pos_emb, mscale, cu_seqlens_kv).squeeze(-2)
 
-        if getattr(self.config, "dsa_indexer_rotate_activation", True):
+        if getattr(self.config, "dsa_indexer_rotate_activation", True) and not defer_rotation:
             q = rotate_activation(q)
             k = rotate_activation(k)
 
@@ -204,7 +206,11 @@ class DSAIndexerFused(MegatronModule):
 
     def forward(self, x, qr, packed_seq_params: Optional[PackedSeqParams] = None):
         """-> ``(index_score_topk [s, topk], topk_indices [s, topk])`` (dsa_fused.py:640-703)."""
-        indexer_query, indexer_key, indexer_weights = self.get_query_key_weight_tensors(x, qr, packed_seq_params)
+        # the rotation moves into the kernel's quantiser when the kernel offers it (head dim 128, device tensors)
+        fuse = (getattr(self.config, "dsa_indexer_rotate_activation", True) and self.index_head_dim == 128
+                and x.is_cuda and getattr(self.indexer_kernel, "supports_fused_rotate", False))
+        indexer_query, indexer_key, indexer_weights = self.get_query_key_weight_tensors(x, qr, packed_seq_params,
+                                                                                        defer_rotation=fuse)
         if packed_seq_params is None:
             indexer_query = indexer_query.squeeze(1).contiguous()
         indexer_key = indexer_key.squeeze(1).contiguous()
@@ -217,6 +223,7 @@ class DSAIndexerFused(MegatronModule):
             self.index_topk,
             chunk_offset=kv_offset,
             packed_seq_params=packed_seq_params,
+            **({"rotate": True} if fuse else {}),
         )
 
 

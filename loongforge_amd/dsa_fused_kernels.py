@@ -166,6 +166,20 @@ def _unscale_indexer_grad(grad, scale_inv):
     return (grad / safe).masked_fill(~usable.expand_as(grad), 0.0)
 
 
+_H128 = {}
+
+
+def _hadamard128(device) -> Tensor:
+    """Sylvester Hadamard matrix of order 128 in fp32 (cached per device)."""
+    key = str(device)
+    if key not in _H128:
+        h = torch.ones(1, 1, dtype=torch.float32, device=device)
+        while h.shape[0] < 128:
+            h = torch.cat([torch.cat([h, h], 1), torch.cat([h, -h], 1)], 0)
+        _H128[key] = h
+    return _H128[key]
+
+
 def _pad_to(x: Tensor, size: int, dim: int) -> Tensor:
     if x.shape[dim] == size:
         return x
@@ -186,7 +200,7 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, index_q: Tensor, index_k: Tensor, weights: Tensor, index_topk: int, chunk_offset: int,
-                packed_seq_params: Optional[PackedSeqParams]):
+                packed_seq_params: Optional[PackedSeqParams], rotate: bool = False):
         assert index_q.ndim == 3 and index_k.ndim == 2 and weights.ndim == 2
         seq_q, head, dim = index_q.size()
         seq_k, _dim = index_k.size()
@@ -199,8 +213,12 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
         assert head <= 64, "the indexer kernel supports at most 64 heads"
         q_p = _pad_to(_pad_to(index_q.to(torch.bfloat16), 128, 2), head_p, 1).contiguous()
         k_p = _pad_to(index_k.to(torch.bfloat16), 128, 1).contiguous()
-        q_fp8, q_scale = ops.quant_rowwise_e4m3(q_p)
-        k_fp8, k_scale = ops.quant_rowwise_e4m3(k_p)
+        # rotate: the Hadamard rotation of the indexer front end is applied here, fused with the
+        # quantiser (a zero-padded head dimension cannot be rotated after padding: 128 only)
+        assert not rotate or dim == 128, "the fused rotation needs head dim 128"
+        quant = ops.rotate_quant_e4m3 if rotate else ops.quant_rowwise_e4m3
+        q_fp8, q_scale = quant(q_p)
+        k_fp8, k_scale = quant(k_p)
 
         if packed_seq_params is None:
             k_start = torch.zeros(seq_q, dtype=torch.int, device=device)
@@ -219,6 +237,7 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
         index_score_topk, topk_indices = ops.indexer_topk(q_fp8, weight_scaled, k_fp8, k_scale, k_start, k_end,
                                                           index_topk, DSAIndexerKernelFunction.sorted_output)
         ctx.softmax_scale = softmax_scale
+        ctx.rotate = rotate
         ctx.index_topk = index_topk
         ctx.shape = (head, dim)
         ctx.in_dtypes = (index_q.dtype, index_k.dtype, weights.dtype)
@@ -236,14 +255,23 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
         d_weights = d_weights * q_scale * ctx.softmax_scale
         d_q = _unscale_indexer_grad(d_q, q_scale)
         d_k = _unscale_indexer_grad(d_k, k_scale)
+        if ctx.rotate:      # the rotation is symmetric and orthogonal up to its scale: its transpose is itself
+            h = _hadamard128(d_q.device)
+            d_q = (d_q @ h) * 128 ** -0.5
+            d_k = (d_k @ h) * 128 ** -0.5
         dq_t, dk_t, dw_t = ctx.in_dtypes
-        return (d_q[:, :head, :dim].to(dq_t), d_k[:, :dim].to(dk_t), d_weights[:, :head].to(dw_t), None, None, None)
+        return (d_q[:, :head, :dim].to(dq_t), d_k[:, :dim].to(dk_t), d_weights[:, :head].to(dw_t), None, None, None,
+                None)
 
 
 class DSAIndexerKernel(torch.nn.Module):
     """``forward(index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params)`` ->
     ``(index_score_topk [sq, topk] fp32, topk_indices [sq, topk] int32)``; reference
-    dsa_fused_kernels.py:2445-2474."""
+    dsa_fused_kernels.py:2445-2474.  ``rotate=True`` (an extension) applies the front end's Hadamard
+    rotation to ``index_q`` / ``index_k`` inside the quantiser kernel instead of before the call."""
 
-    def forward(self, index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params):
-        return DSAIndexerKernelFunction.apply(index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params)
+    supports_fused_rotate = True
+
+    def forward(self, index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params, rotate=False):
+        return DSAIndexerKernelFunction.apply(index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params,
+                                              rotate)

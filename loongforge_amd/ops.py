@@ -61,6 +61,49 @@ def quant_rowwise_e4m3(x: torch.Tensor, eps: float = 1e-12, pow2: bool = True):
     return x8.view(_FP8), scale_inv
 
 
+@torch.library.custom_op("dsa::rotate_quant_e4m3", mutates_args=())
+def _rotate_quant_op(x: torch.Tensor, eps: float, pow2: bool, want_payload: bool,
+                     want_rotated: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _need_gpu(x)
+    if x.dtype != torch.bfloat16:
+        raise ValueError("rotate_quant_e4m3 expects bf16 input, got %s" % x.dtype)
+    if x.shape[-1] != 128:
+        raise ValueError("rotate_quant_e4m3 rotates rows of 128 elements, got %d" % x.shape[-1])
+    if not (want_payload or want_rotated):
+        raise ValueError("rotate_quant_e4m3: no output requested")
+    x = _c(x)
+    rows = x.numel() // 128
+    x8 = torch.empty(x.shape if want_payload else (0,), dtype=torch.uint8, device=x.device)
+    scale_inv = torch.empty(x.shape[:-1] if want_payload else (0,), dtype=torch.float32, device=x.device)
+    y = torch.empty(x.shape if want_rotated else (0,), dtype=torch.bfloat16, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        _lib.check(lib.dsa_rotate_quant_e4m3(x.data_ptr(), rows, 128, x8.data_ptr() if want_payload else None,
+                                             scale_inv.data_ptr() if want_payload else None,
+                                             y.data_ptr() if want_rotated else None, float(eps), int(pow2), _stream(x)),
+                   "dsa_rotate_quant_e4m3")
+    return x8, scale_inv, y
+
+
+@_rotate_quant_op.register_fake
+def _(x, eps, pow2, want_payload, want_rotated):
+    return (x.new_empty(x.shape if want_payload else (0,), dtype=torch.uint8),
+            x.new_empty(x.shape[:-1] if want_payload else (0,), dtype=torch.float32),
+            x.new_empty(x.shape if want_rotated else (0,), dtype=torch.bfloat16))
+
+
+def rotate_quant_e4m3(x: torch.Tensor, eps: float = 1e-12, pow2: bool = True, return_rotated: bool = False):
+    """Hadamard rotation (x 128^-0.5, rounded to bf16) fused with :func:`quant_rowwise_e4m3`:
+    bf16 ``[..., 128]`` -> (fp8 payload, ``scale_inv``[, rotated bf16])."""
+    x8, scale_inv, y = _rotate_quant_op(x, eps, pow2, True, return_rotated)
+    return (x8.view(_FP8), scale_inv, y) if return_rotated else (x8.view(_FP8), scale_inv)
+
+
+def rotate_bf16(x: torch.Tensor):
+    """Hadamard rotation of bf16 rows of 128 (x 128^-0.5), the kernel form of ``rotate_activation``."""
+    return _rotate_quant_op(x, 1e-12, True, False, True)[2]
+
+
 def _as_u8(t: torch.Tensor) -> torch.Tensor:
     if t.dtype == _FP8:
         return t.view(torch.uint8)

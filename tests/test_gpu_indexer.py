@@ -186,3 +186,56 @@ def test_topk_rule_on_crafted_rows(gpu, kind, K, sorted_out):
             assert torch.equal(torch.sort(got).values, torch.sort(exp_ids).values), (kind, K, i)
             assert torch.equal(sc[i][ids[i] >= 0], row[got])
         assert (ids[i, kk:] == -1).all() and torch.isinf(sc[i, kk:]).all() and (sc[i, kk:] < 0).all()
+
+
+def test_fused_rotation_and_quantiser(gpu):
+    """rotate_quant_e4m3 against the unfused sequence rotate_activation -> quantiser: the rotated bf16
+    values agree to one bf16 step (the fp32 sums are taken in a different order), payload and scale
+    are exactly the quantisation of the kernel's own rotated values, and the rotation is an involution."""
+    from loongforge_amd import ops
+    from loongforge_amd.dsa_fused import rotate_activation
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1000, 7, 128, generator=g).to(torch.bfloat16)
+    x[5] = 0
+    xd = x.to(gpu)
+    x8, sinv, y = ops.rotate_quant_e4m3(xd, return_rotated=True)
+    ref = rotate_activation(x)                                       # fp32 product with the Hadamard matrix on the CPU
+    err = (y.cpu().float() - ref.float()).abs()
+    assert (err <= 2.0 ** -7 * ref.float().abs() + 1e-30).all()      # at most one bf16 step
+    assert (err == 0).float().mean().item() > 0.98
+    r8, rs = O.quant_rowwise_e4m3(y.cpu())
+    assert torch.equal(x8.cpu().view(torch.uint8), r8.view(torch.uint8)) and torch.equal(sinv.cpu(), rs)
+    x8b, sinvb = ops.rotate_quant_e4m3(xd)
+    assert torch.equal(x8b.view(torch.uint8), x8.view(torch.uint8)) and torch.equal(sinvb, sinv)
+    assert torch.equal(ops.rotate_bf16(xd), y)
+    back = ops.rotate_bf16(y).float().cpu()                          # H.H = 128 I: rotating twice returns x
+    assert (back - x.float()).abs().max().item() <= 2.0 ** -6 * x.float().abs().max().item()
+
+
+def test_indexer_kernel_with_fused_rotation_matches_rotating_first(gpu):
+    """DSAIndexerKernel(rotate=True) == DSAIndexerKernel on pre-rotated inputs: same scores and ids, and
+    gradients that agree with autograd through rotate_activation."""
+    from loongforge_amd.dsa_fused import rotate_activation
+    from loongforge_amd.dsa_fused_kernels import DSAIndexerKernel
+
+    S, Hi, K = 512, 64, 128
+    iq, ik, w = O.make_indexer_inputs(S, Hi, 128, seed=11)
+    kern = DSAIndexerKernel()
+    q1, k1, w1 = (t.to(gpu).requires_grad_(True) for t in (iq, ik, w))
+    sc1, id1 = kern(q1, k1, w1, K, 0, None, rotate=True)
+    q2, k2, w2 = (t.to(gpu).requires_grad_(True) for t in (iq, ik, w))
+    sc2, id2 = kern(rotate_activation(q2), rotate_activation(k2), w2, K, 0, None)
+    fin = torch.isfinite(sc2)
+    assert torch.equal(torch.isfinite(sc1), fin)
+    # a bf16 step in a few rotated values moves a logit by a few 1e-3 of the row's scale
+    tol = 5e-3 * sc2[fin].abs().max().item()
+    assert (sc1[fin] - sc2[fin]).abs().max().item() <= tol
+    same = (torch.sort(id1, 1).values == torch.sort(id2, 1).values).float().mean().item()
+    assert same > 0.99
+    gsc = torch.randn(S, K, generator=torch.Generator().manual_seed(12)).to(gpu)
+    torch.where(fin, sc1, torch.zeros_like(sc1)).mul(gsc).sum().backward()
+    torch.where(fin, sc2, torch.zeros_like(sc2)).mul(gsc).sum().backward()
+    for a, b in ((q1.grad, q2.grad), (k1.grad, k2.grad), (w1.grad, w2.grad)):
+        scale = b.float().abs().max().item()
+        assert (a.float() - b.float()).abs().max().item() <= 3e-2 * scale
