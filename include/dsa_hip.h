@@ -124,6 +124,19 @@ int dsa_sparse_mla_fwd(const void* q, const void* kv, const int32_t* ids, int S,
                        void* p_out, int p_out_f32, void* stream);
 
 /*
+ * The same with a per-head attention-sink logit (attn_sink [H] f32, NULL = none): the softmax
+ * denominator gains the term exp(attn_sink[h]), which has no value row, so
+ *   P = exp(s * sm_scale) / (sum_t exp(s * sm_scale) + exp(attn_sink[h]))   and lse includes the sink;
+ * a query without valid slots gets lse = attn_sink[h] and a zero output row.  This is the
+ * `attn_sink` argument of flash_mla_sparse_fwd at dsa_fused_kernels.py:2040-2057; its math is the
+ * torch formulation at loongforge/models/foundation/deepseek_v4/deepseek_v4_csa.py:571-579.
+ * dsa_sparse_mla_bwd needs no sink argument: the sink enters dQ / dKV only through lse.
+ */
+int dsa_sparse_mla_fwd_sink(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv,
+                            int K, int q_start, float sm_scale, int d_v, void* out, float* lse,
+                            void* p_out, int p_out_f32, const float* attn_sink, void* stream);
+
+/*
  * Sparse MQA-MLA attention backward: dQ and dKV of dsa_sparse_mla_fwd given dO, the saved out and
  * natural-log lse.  dKV is accumulated in fp32 in a fixed order (bit-reproducible, no float
  * atomics) and returned as bf16.  Replaces flash_mla_bwd.flash_mla_sparse_bwd /

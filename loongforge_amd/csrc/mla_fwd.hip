@@ -66,7 +66,7 @@ template <int STAGES, int POUT, bool EXACT>   // POUT: 0 none, 1 bf16, 2 f32
 __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
     __bf16* __restrict__ out, float* __restrict__ lse, void* __restrict__ p_out,
-    int S, int H, int Skv, int K, int q_start, float sm_scale) {
+    int S, int H, int Skv, int K, int q_start, float sm_scale, const float* __restrict__ sink) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, g = lane >> 5;
@@ -327,13 +327,24 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
   }
 
   // ---- epilogue: normalise, write out[i,h,:] and lse[i,h] ---------------------------------
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   if (!EXACT && __ballot(overflow) != 0ull) {
     // leave the query to the exact pass (it rewrites out, lse and p_out of all heads)
     if (lane == 0 && wave * 32 < H) ((unsigned*)lse)[(size_t)qi * H + wave * 32] = LSE_REDO_MARK;
     return;
   }
+  float o_scale = 1.0f;
+  if (sink) {
+    // per-head sink logit: one more term exp(sink) in the denominator, with no value row.  The
+    // reference point moves to max(reference, sink) so that neither term can overflow; a query
+    // without any valid slot ends with lse = sink and a zero output row.
+    const float sk2 = sink[head_ok ? h : 0] * LOG2E;
+    const float nm = fmaxf(m_ref, sk2);
+    o_scale = exp2f(m_ref - nm);
+    l_tot = l_tot * o_scale + exp2f(sk2 - nm);
+    m_ref = nm;
+  }
+  const float inv = l_tot > 0.f ? o_scale / l_tot : 0.f;
   if (head_ok) {
     if (g == 0) lse[(size_t)qi * H + h] = l_tot > 0.f ? (m_ref + log2f(l_tot)) * 0.6931471805599453f : INFINITY;
     unsigned short* op = (unsigned short*)out + ((size_t)qi * H + h) * DV + 4 * g;
@@ -350,7 +361,7 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
 
 template <int STAGES>
 int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K, int q_start,
-               float sm_scale, void* out, float* lse, void* p_out, int p_out_f32, hipStream_t st) {
+               float sm_scale, void* out, float* lse, void* p_out, int p_out_f32, const float* sink, hipStream_t st) {
   const size_t smem = (size_t)STAGES * TILE_BYTES + (size_t)K * 4 + (size_t)(K / BI) * 8 + 16;   // ids, tile masks, tile list, counters
   if (smem > 160 * 1024) return -1;
   dim3 grid(S), block(256);
@@ -359,8 +370,8 @@ int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, 
     auto kern2 = mla_fwd_kernel<STAGES, P, true>; \
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2; \
     if (hipFuncSetAttribute((const void*)kern2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2; \
-    kern<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale); \
-    kern2<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale); \
+    kern<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink); \
+    kern2<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink); \
   } while (0)
   if (!p_out) DSA_FWD_LAUNCH(0);
   else if (!p_out_f32) DSA_FWD_LAUNCH(1);
@@ -371,24 +382,30 @@ int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, 
 
 }  // namespace
 
-extern "C" int dsa_sparse_mla_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K,
-                                  int q_start, float sm_scale, int d_v, void* out, float* lse, void* p_out,
-                                  int p_out_f32, void* stream) {
+extern "C" int dsa_sparse_mla_fwd_sink(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K,
+                                       int q_start, float sm_scale, int d_v, void* out, float* lse, void* p_out,
+                                       int p_out_f32, const float* attn_sink, void* stream) {
   DSA_REQUIRE(d_v == DV, "dsa_sparse_mla_fwd: only d_v = 512 (d_qk = 576) is supported, got d_v = %d", d_v);
   DSA_REQUIRE(S >= 0 && Skv > 0, "dsa_sparse_mla_fwd: bad sequence sizes S=%d Skv=%d", S, Skv);
   DSA_REQUIRE(H > 0 && H <= 128 && H % 32 == 0, "dsa_sparse_mla_fwd: head count must be 32, 64, 96 or 128, got %d", H);
   DSA_REQUIRE(K > 0 && K % 64 == 0, "dsa_sparse_mla_fwd: top-k must be a positive multiple of 64, got %d", K);
   DSA_REQUIRE((size_t)Skv * DQK * 2 <= 0xffffffffull, "dsa_sparse_mla_fwd: kv larger than 4 GiB is not supported");
   DSA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)kv % 16) == 0 && ((uintptr_t)out % 8) == 0 &&
-              ((uintptr_t)p_out % 16) == 0, "dsa_sparse_mla_fwd: misaligned pointer");
+              ((uintptr_t)p_out % 16) == 0 && ((uintptr_t)attn_sink % 4) == 0, "dsa_sparse_mla_fwd: misaligned pointer");
   if (S == 0) return DSA_OK;
   hipStream_t st = (hipStream_t)stream;
   int rc;
-  if (K <= 2048) rc = launch_fwd<4>(q, kv, ids, S, H, Skv, K, q_start, sm_scale, out, lse, p_out, p_out_f32, st);
-  else if (K <= 8192) rc = launch_fwd<3>(q, kv, ids, S, H, Skv, K, q_start, sm_scale, out, lse, p_out, p_out_f32, st);
+  if (K <= 2048) rc = launch_fwd<4>(q, kv, ids, S, H, Skv, K, q_start, sm_scale, out, lse, p_out, p_out_f32, attn_sink, st);
+  else if (K <= 8192) rc = launch_fwd<3>(q, kv, ids, S, H, Skv, K, q_start, sm_scale, out, lse, p_out, p_out_f32, attn_sink, st);
   else rc = -1;
   DSA_REQUIRE(rc != -1, "dsa_sparse_mla_fwd: top-k %d exceeds the supported maximum 8192", K);
   if (rc == -2) DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_fwd: cannot reserve LDS");
   DSA_CHECK_LAUNCH("dsa_sparse_mla_fwd");
   return DSA_OK;
+}
+
+extern "C" int dsa_sparse_mla_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K,
+                                  int q_start, float sm_scale, int d_v, void* out, float* lse, void* p_out,
+                                  int p_out_f32, void* stream) {
+  return dsa_sparse_mla_fwd_sink(q, kv, ids, S, H, Skv, K, q_start, sm_scale, d_v, out, lse, p_out, p_out_f32, nullptr, stream);
 }

@@ -52,21 +52,32 @@ def padded_flashinfer_topk(logits, topk, sk, *, sorted=True):
 class DSADotProductAttentionFunction(torch.autograd.Function):
     """Sparse MLA attention over the selected latent rows (forward and backward on the HIP kernels).
 
-    Same argument list as the reference (dsa_fused_kernels.py:2006-2021).  ``topk_length``,
-    ``attn_sink`` and ``window_size`` belong to a different attention variant and must keep their
-    defaults.
+    Same argument list as the reference (dsa_fused_kernels.py:2006-2021).  ``attn_sink`` ([h_q] or a
+    divisor of it, expanded as at :2040-2046) adds a per-head sink term to the softmax denominator;
+    ``topk_length`` ([s_q] int32) keeps only the first ``topk_length[i]`` slots of query ``i``.  No
+    gradient is returned for ``attn_sink`` (the reference returns none either, :2112).
+    ``window_size`` belongs to a different attention variant and must keep its default.
     """
 
     @staticmethod
     def forward(ctx, q, kv, indices, chunk_offset=0, sm_scale=None, d_v=512, return_p_out=False,
                 packed_seq_params=None, topk_length=None, attn_sink=None, window_size=0, fast_mode=False):
-        if topk_length is not None or attn_sink is not None or window_size not in (0, None):
-            raise NotImplementedError("topk_length / attn_sink / window_size are not supported by this build")
+        if window_size not in (0, None):
+            raise NotImplementedError("window_size is not supported by this build")
         # q [sq, n, d]; kv [skv, 1, d]; indices [sq, 1, topk]
         sq = q.size(0)
         kv2 = kv.reshape(kv.shape[0], kv.shape[-1])
         ids = indices.reshape(sq, indices.shape[-1])
-        out, lse, p_out = ops.sparse_mla_fwd(q, kv2, ids, chunk_offset, sm_scale, d_v, return_p_out)
+        if topk_length is not None:
+            slot = torch.arange(ids.shape[-1], device=ids.device)
+            ids = torch.where(slot[None, :] < topk_length.reshape(sq, 1).to(ids.device), ids, torch.full_like(ids, -1))
+        if attn_sink is not None:
+            h_q = q.size(1)
+            if attn_sink.numel() != h_q:
+                attn_sink = attn_sink.flatten().repeat_interleave(h_q // attn_sink.numel())
+            attn_sink = attn_sink.contiguous().view(h_q).float()
+        out, lse, p_out = ops.sparse_mla_fwd(q, kv2, ids, chunk_offset, sm_scale, d_v, return_p_out,
+                                             attn_sink=attn_sink)
         ctx.save_for_backward(q, kv, ids, out, lse)
         ctx.sm_scale = sm_scale
         ctx.chunk_offset = chunk_offset

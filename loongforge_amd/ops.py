@@ -278,10 +278,15 @@ def _check_mla(q, kv, ids):
 
 @torch.library.custom_op("dsa::sparse_mla_fwd", mutates_args=())
 def _mla_fwd_op(q: torch.Tensor, kv: torch.Tensor, ids: torch.Tensor, q_start: int, sm_scale: float, d_v: int,
-                p_out_mode: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                p_out_mode: int, attn_sink: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     _check_mla(q, kv, ids)
     q, kv, ids = _c(q), _c(kv), _c(ids.int())
     S, H, _ = q.shape
+    if attn_sink is not None:
+        _need_gpu(attn_sink)
+        if attn_sink.numel() != H:
+            raise ValueError("attn_sink must hold one logit per head (%d), got %d" % (H, attn_sink.numel()))
+        attn_sink = _c(attn_sink.float().reshape(H))
     K = ids.shape[1]
     out = torch.empty(S, H, d_v, dtype=torch.bfloat16, device=q.device)
     lse = torch.empty(S, H, dtype=torch.float32, device=q.device)
@@ -291,27 +296,30 @@ def _mla_fwd_op(q: torch.Tensor, kv: torch.Tensor, ids: torch.Tensor, q_start: i
         p_out = torch.empty(S, H, K, dtype=torch.float32 if p_out_mode == 2 else torch.bfloat16, device=q.device)
     lib = _lib.load()
     with torch.cuda.device(q.device):
-        _lib.check(lib.dsa_sparse_mla_fwd(q.data_ptr(), kv.data_ptr(), ids.data_ptr(), S, H, kv.shape[0], K,
-                                          int(q_start), float(sm_scale), int(d_v), out.data_ptr(), lse.data_ptr(),
-                                          p_out.data_ptr() if p_out_mode else None, int(p_out_mode == 2), _stream(q)),
+        _lib.check(lib.dsa_sparse_mla_fwd_sink(q.data_ptr(), kv.data_ptr(), ids.data_ptr(), S, H, kv.shape[0], K,
+                                               int(q_start), float(sm_scale), int(d_v), out.data_ptr(), lse.data_ptr(),
+                                               p_out.data_ptr() if p_out_mode else None, int(p_out_mode == 2),
+                                               attn_sink.data_ptr() if attn_sink is not None else None, _stream(q)),
                    "dsa_sparse_mla_fwd")
     return out, lse, p_out
 
 
 @_mla_fwd_op.register_fake
-def _(q, kv, ids, q_start, sm_scale, d_v, p_out_mode):
+def _(q, kv, ids, q_start, sm_scale, d_v, p_out_mode, attn_sink=None):
     S, H, _ = q.shape
     p = q.new_empty(0) if p_out_mode == 0 else q.new_empty(S, H, ids.shape[1], dtype=torch.float32 if p_out_mode == 2 else torch.bfloat16)
     return q.new_empty(S, H, d_v), q.new_empty(S, H, dtype=torch.float32), p
 
 
 def sparse_mla_fwd(q, kv, ids, q_start: int = 0, sm_scale: Optional[float] = None, d_v: int = 512,
-                   return_p_out: bool = False, p_out_dtype: torch.dtype = torch.bfloat16):
-    """(out bf16 [S,H,d_v], natural-log lse fp32 [S,H], p_out or None)."""
+                   return_p_out: bool = False, p_out_dtype: torch.dtype = torch.bfloat16,
+                   attn_sink: Optional[torch.Tensor] = None):
+    """(out bf16 [S,H,d_v], natural-log lse fp32 [S,H], p_out or None).  ``attn_sink`` [H]: per-head
+    sink logit added to the softmax denominator (and to lse)."""
     if sm_scale is None:
         sm_scale = q.shape[-1] ** -0.5
     mode = 0 if not return_p_out else (2 if p_out_dtype == torch.float32 else 1)
-    out, lse, p_out = _mla_fwd_op(q, kv, ids, int(q_start), float(sm_scale), int(d_v), mode)
+    out, lse, p_out = _mla_fwd_op(q, kv, ids, int(q_start), float(sm_scale), int(d_v), mode, attn_sink)
     return out, lse, (p_out if return_p_out else None)
 
 

@@ -22,9 +22,12 @@ topk_select             pinned: torch.sort brute force + set invariants.
                         (closed wheel); order inside a row is not part of the contract.
 sparse_mla_fwd          pinned: equals dense causal MQA (SDPA) when top-k covers the prefix;
                         brute-force fp64 loops in the general case; invariants.
+                        attn_sink: the sink softmax written out as loops after the open torch
+                        text at deepseek_v4_csa.py:571-579, plus the sink-share identity.
                         unpinned detail: p_out dtype / fill value of the closed flash_mla_fwd.
 sparse_mla_bwd          pinned: torch.autograd through the forward restatement, gradcheck in
-                        fp64, dense-attention gradients (SDPA autograd) in the covering case.
+                        fp64, dense-attention gradients (SDPA autograd) in the covering case;
+                        finite differences with a sink.
 attn_dist, indexer_kl_loss   pinned: closed forms, F.kl_div, analytic special cases.
 indexer_bwd             pinned: autograd through the gathered logits; finite differences.
                         unpinned detail: duplicate / out-of-window id handling of the closed
@@ -219,6 +222,7 @@ def sparse_mla_fwd(
     d_v: int = 512,
     dtype: torch.dtype = torch.float32,
     chunk: int = 64,
+    attn_sink: Optional[torch.Tensor] = None,   # [h] per-head sink logit
 ):
     """Gather formulation of sparse MQA-MLA attention.
 
@@ -227,6 +231,9 @@ def sparse_mla_fwd(
     Returns ``out [sq,h,d_v]``, natural-log ``lse [sq,h]`` (+inf for rows without a valid slot,
     whose ``out`` is 0) and ``p_out [sq,h,K]`` = raw (unscaled) logits, -inf on invalid slots
     (consumer applies ``* sm_scale`` and softmax: dsa_fused_kernels.py:1884-1890).
+    ``attn_sink``: the denominator gains ``exp(attn_sink[h])`` (deepseek_v4_csa.py:571-579): the
+    sink is one more logit without a value row, so ``lse`` includes it and an empty row has
+    ``lse = attn_sink`` and ``out = 0``.
     Differentiable in q and kv.
     """
     sq, h, dqk = q.shape
@@ -243,7 +250,11 @@ def sparse_mla_fwd(
         sc = torch.einsum("mhd,mkd->mhk", qf[s:e], kvg)        # raw logits
         sc = sc.masked_fill(~valid[s:e].unsqueeze(1), NEG_INF)
         z = sc * sm_scale
-        lse = torch.logsumexp(z, dim=-1)                       # -inf for empty rows
+        if attn_sink is not None:
+            zs = torch.cat([z, attn_sink.to(dtype).view(1, h, 1).expand(e - s, h, 1)], dim=-1)
+            lse = torch.logsumexp(zs, dim=-1)
+        else:
+            lse = torch.logsumexp(z, dim=-1)                   # -inf for empty rows
         empty = torch.isinf(lse) & (lse < 0)
         p = torch.exp(z - lse.masked_fill(empty, 0.0).unsqueeze(-1))
         p = p.masked_fill(empty.unsqueeze(-1), 0.0)
@@ -253,14 +264,14 @@ def sparse_mla_fwd(
     return torch.cat(outs), torch.cat(lses), torch.cat(pouts)
 
 
-def sparse_mla_bwd(q, kv, idx, dout, q_start=0, sm_scale=None, d_v=512, dtype=torch.float32):
+def sparse_mla_bwd(q, kv, idx, dout, q_start=0, sm_scale=None, d_v=512, dtype=torch.float32, attn_sink=None):
     """dQ, dKV by autograd through :func:`sparse_mla_fwd` -- exactly what the reference's own
     check does (ops/tilelang_ops/sparse_mla_bwd.py:310-319).  The closed form it must agree
     with is in that file's kernel, :176-231: ``dS = P*(dP - Delta)*scale``, ``dQ = dS.KV``,
     ``dKV[idx] += dS^T.Q (+ P^T.dO on the first d_v dims)``."""
     qd = q.detach().to(dtype).requires_grad_(True)
     kvd = kv.detach().to(dtype).requires_grad_(True)
-    out, _, _ = sparse_mla_fwd(qd, kvd, idx, q_start, sm_scale, d_v, dtype=dtype)
+    out, _, _ = sparse_mla_fwd(qd, kvd, idx, q_start, sm_scale, d_v, dtype=dtype, attn_sink=attn_sink)
     out.backward(dout.to(dtype))
     return qd.grad, kvd.grad
 

@@ -46,6 +46,19 @@ def test_dot_product_attention_layouts_and_autograd(gpu):
         attn(q.unsqueeze(1), kv.unsqueeze(1), ids.unsqueeze(0), 0, AttnMaskType.no_mask)
     with pytest.raises(NotImplementedError):
         attn(q.unsqueeze(1), kv.unsqueeze(1), ids.unsqueeze(0), 0, None, window_size=4)
+    # topk_length keeps a prefix of each query's slots; attn_sink ([h] or a divisor of it) joins the denominator
+    tl = torch.randint(0, 101, (150,), generator=torch.Generator().manual_seed(4), dtype=torch.int32)
+    sink = torch.linspace(-2, 2, 64)
+    q.grad = kv.grad = None
+    out3 = attn(q.unsqueeze(1), kv.unsqueeze(1), ids.unsqueeze(0), 0, None, topk_length=tl.to(gpu), attn_sink=sink.to(gpu))
+    cut = torch.where(torch.arange(inp.idx.shape[1])[None, :] < tl[:, None], inp.idx, torch.full_like(inp.idx, -1))
+    sink_h = sink.repeat_interleave(2)
+    ro3, _, _ = O.sparse_mla_fwd(inp.q, inp.kv, cut, 0, inp.sm_scale, 512, attn_sink=sink_h)
+    assert_close(out3[0], ro3, "out with topk_length and sink")
+    out3.backward(inp.dout.to(gpu).unsqueeze(0))
+    rdq3, rdkv3 = O.sparse_mla_bwd(inp.q, inp.kv, cut, inp.dout, 0, inp.sm_scale, 512, attn_sink=sink_h)
+    assert_close(q.grad, rdq3, "dq with topk_length and sink", scale_aware=True)
+    assert_close(kv.grad, rdkv3, "dkv with topk_length and sink", scale_aware=True)
 
 
 def test_sparse_mla_bwd_interface_signature(gpu):

@@ -113,6 +113,52 @@ def test_backward_against_oracle_and_deterministic(gpu, S, H, K, q_start, skv, s
     assert torch.equal(dq, dq2) and torch.equal(dkv, dkv2)          # bit-identical
 
 
+def test_forward_and_backward_with_attention_sink(gpu):
+    from loongforge_amd import ops
+
+    S, H, K, q_start = 200, 128, 128, 40
+    inp = O.make_mla_inputs(S, H, K, seed=7, skv=300, q_start=q_start)
+    idx = inp.idx.clone()
+    idx[9, :] = -1                                                  # a row with only the sink
+    g = torch.Generator().manual_seed(3)
+    sink = torch.randn(H, generator=g) * 3.0
+    sink[0], sink[1], sink[2] = 60.0, -60.0, 0.0                    # dominant, negligible, neutral
+    q, kv, ids, do = inp.q.to(gpu), inp.kv.to(gpu), idx.to(gpu), inp.dout.to(gpu)
+    out, lse, _ = ops.sparse_mla_fwd(q, kv, ids, q_start, inp.sm_scale, attn_sink=sink.to(gpu))
+    ro, rl, _ = O.sparse_mla_fwd(inp.q, inp.kv, idx, q_start, inp.sm_scale, 512, attn_sink=sink)
+    assert_close(out, ro, "out")
+    assert torch.isfinite(lse).all()
+    assert (lse.cpu() - rl).abs().max().item() < 1e-4
+    assert (lse[9].cpu() - sink).abs().max().item() < 1e-5 and out[9].abs().max().item() == 0
+    # without a sink the same call is unchanged by the extra argument
+    o0, l0, _ = ops.sparse_mla_fwd(q, kv, ids, q_start, inp.sm_scale)
+    o1, l1, _ = ops.sparse_mla_fwd(q, kv, ids, q_start, inp.sm_scale, attn_sink=None)
+    assert torch.equal(o0, o1) and torch.equal(l0, l1)
+    dq, dkv = ops.sparse_mla_bwd(q, kv, out, do, ids, lse, q_start, inp.sm_scale)
+    rdq, rdkv = O.sparse_mla_bwd(inp.q, inp.kv, idx, inp.dout, q_start, inp.sm_scale, 512, attn_sink=sink)
+    assert_close(dq, rdq, "dq", scale_aware=True)
+    assert_close(dkv, rdkv, "dkv", scale_aware=True)
+
+
+def test_sink_survives_the_exact_pass(gpu):
+    # a late dominant key sends the query through the second (exact-maximum) pass; the sink term
+    # must be applied there as well
+    from loongforge_amd import ops
+
+    inp = O.make_mla_inputs(80, 128, 64, seed=6)
+    kv = inp.kv.clone().float()
+    kv[70] = inp.q[79, 0].float() * 40.0
+    kv = kv.to(torch.bfloat16)
+    idx = inp.idx.clone()
+    idx[79, 63] = 70
+    sink = torch.linspace(-4, 4, 128)
+    sink[0] = 1567.0                                 # comparable with the dominant logit of head 0 (about 1568)
+    out, lse, _ = ops.sparse_mla_fwd(inp.q.to(gpu), kv.to(gpu), idx.to(gpu), 0, inp.sm_scale, attn_sink=sink.to(gpu))
+    ro, rl, _ = O.sparse_mla_fwd(inp.q, kv, idx, 0, inp.sm_scale, 512, attn_sink=sink)
+    assert_close(out, ro, "out", atol=4e-2)
+    assert ((lse.cpu() - rl).abs() / rl.abs().clamp_min(1)).max().item() < 1e-3
+
+
 def test_backward_chunked_workspace_through_the_c_abi(gpu):
     """A workspace too small for all queries at once makes the library walk the queries in chunks;
     the result must not change."""

@@ -65,6 +65,67 @@ def test_fwd_brute_force_general_case_with_invalid_ids():
             assert math.isclose(lse[i, hh].item(), m + math.log(tot), rel_tol=1e-12)
 
 
+def test_fwd_with_sink_matches_the_sink_softmax_written_out():
+    # deepseek_v4_csa.py:571-579: weights = exp(s - m) / (sum exp(s - m) + exp(sink - m)) with
+    # m = max(max s, sink); the sink has no value row.  Written here as plain loops.
+    sq, h, dqk, dv, K = 18, 3, 12, 8, 6
+    q, kv, idx = _inputs(sq, h, K, dqk, seed=11, q_start=2, skv=24)
+    idx = idx.clone()
+    idx[4, :] = -1                                           # no valid slot: only the sink remains
+    idx[5, 1] = -1
+    sink = torch.tensor([-1.3, 0.4, 7.0], dtype=torch.float64)
+    sm = 0.29
+    out, lse, _ = O.sparse_mla_fwd(q, kv, idx, 2, sm, dv, dtype=torch.float64, attn_sink=sink)
+    for i in range(sq):
+        for hh in range(h):
+            sc, rows = [], []
+            for t in range(K):
+                j = int(idx[i, t])
+                if j != -1 and 0 <= j < 24 and j <= 2 + i:
+                    sc.append(float(np.dot(q[i, hh].numpy(), kv[j].numpy())) * sm)
+                    rows.append(j)
+            m = max(sc + [float(sink[hh])])
+            den = sum(math.exp(s - m) for s in sc) + math.exp(float(sink[hh]) - m)
+            ref = np.zeros(dv)
+            for s, j in zip(sc, rows):
+                ref += math.exp(s - m) / den * kv[j, :dv].numpy()
+            np.testing.assert_allclose(out[i, hh].numpy(), ref, rtol=1e-10, atol=1e-12)
+            assert math.isclose(lse[i, hh].item(), m + math.log(den), rel_tol=1e-12, abs_tol=1e-12)
+    assert torch.equal(lse[4], sink) and out[4].abs().max() == 0
+    # a sink far below every logit changes nothing; the weights of a row sum to 1 - sink share
+    o0, l0, _ = O.sparse_mla_fwd(q, kv, idx, 2, sm, dv, dtype=torch.float64)
+    o1, l1, _ = O.sparse_mla_fwd(q, kv, idx, 2, sm, dv, dtype=torch.float64, attn_sink=torch.full((3,), -800.0, dtype=torch.float64))
+    ok = torch.isfinite(l0)
+    torch.testing.assert_close(o1[ok], o0[ok], rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(l1[ok], l0[ok], rtol=1e-12, atol=1e-12)
+    share = 1 - torch.exp(sink[None, :] - lse)
+    torch.testing.assert_close(out[ok], o0[ok] * share[ok].unsqueeze(-1), rtol=1e-10, atol=1e-12)
+
+
+def test_bwd_with_sink_matches_finite_differences():
+    sq, h, dqk, dv, K = 6, 2, 8, 4, 4
+    q, kv, idx = _inputs(sq, h, K, dqk, seed=13)
+    sink = torch.tensor([0.3, -0.8], dtype=torch.float64)
+    g = torch.Generator().manual_seed(5)
+    dout = torch.randn(sq, h, dv, generator=g, dtype=torch.float64)
+    dq, dkv = O.sparse_mla_bwd(q, kv, idx, dout, 0, 0.4, dv, dtype=torch.float64, attn_sink=sink)
+
+    def f(q_, kv_):
+        return (O.sparse_mla_fwd(q_, kv_, idx, 0, 0.4, dv, dtype=torch.float64, attn_sink=sink)[0] * dout).sum().item()
+
+    eps = 1e-6
+    for (i, hh, d) in [(0, 0, 0), (3, 1, 5), (5, 0, 7)]:
+        qp, qm = q.clone(), q.clone()
+        qp[i, hh, d] += eps
+        qm[i, hh, d] -= eps
+        assert math.isclose((f(qp, kv) - f(qm, kv)) / (2 * eps), dq[i, hh, d].item(), rel_tol=1e-6, abs_tol=1e-8)
+    for (j, d) in [(0, 0), (2, 3), (4, 6)]:
+        kp, km = kv.clone(), kv.clone()
+        kp[j, d] += eps
+        km[j, d] -= eps
+        assert math.isclose((f(q, kp) - f(q, km)) / (2 * eps), dkv[j, d].item(), rel_tol=1e-6, abs_tol=1e-8)
+
+
 def test_fwd_is_invariant_to_slot_permutation():
     q, kv, idx = _inputs(16, 2, 8, seed=5)
     perm = torch.randperm(8, generator=torch.Generator().manual_seed(9))
