@@ -131,10 +131,14 @@ int dsa_sparse_mla_fwd(const void* q, const void* kv, const int32_t* ids, int S,
  * `attn_sink` argument of flash_mla_sparse_fwd at dsa_fused_kernels.py:2040-2057; its math is the
  * torch formulation at loongforge/models/foundation/deepseek_v4/deepseek_v4_csa.py:571-579.
  * dsa_sparse_mla_bwd needs no sink argument: the sink enters dQ / dKV only through lse.
+ * p_out_skip (a multiple of 32, < K; 0 = none): p_out leaves out the first p_out_skip slots of every
+ * query and is [S,H,K - p_out_skip]; attention itself still runs over all K slots.  This is the
+ * `window_size` argument of the same call (:2058): the DeepSeek-V4 caller puts its sliding-window
+ * keys in the leading slots and documents the resulting p_out width at deepseek_v4_csa.py:2341-2346.
  */
-int dsa_sparse_mla_fwd_sink(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv,
-                            int K, int q_start, float sm_scale, int d_v, void* out, float* lse,
-                            void* p_out, int p_out_f32, const float* attn_sink, void* stream);
+int dsa_sparse_mla_fwd_ex(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv,
+                          int K, int q_start, float sm_scale, int d_v, void* out, float* lse,
+                          void* p_out, int p_out_f32, const float* attn_sink, int p_out_skip, void* stream);
 
 /*
  * Sparse MQA-MLA attention backward: dQ and dKV of dsa_sparse_mla_fwd given dO, the saved out and

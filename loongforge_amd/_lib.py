@@ -25,7 +25,7 @@ SIGNATURES = {
     "dsa_indexer_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "dsa_indexer_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
     "dsa_sparse_mla_fwd": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _i, _vp]),
-    "dsa_sparse_mla_fwd_sink": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _i, _vp, _vp]),
+    "dsa_sparse_mla_fwd_ex": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _i, _vp, _i, _vp]),
     "dsa_sparse_mla_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "dsa_sparse_mla_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _sz, _vp]),
     "dsa_sparse_mla_bwd_profile": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _sz, _vp,

@@ -66,7 +66,7 @@ template <int STAGES, int POUT, bool EXACT>   // POUT: 0 none, 1 bf16, 2 f32
 __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
     __bf16* __restrict__ out, float* __restrict__ lse, void* __restrict__ p_out,
-    int S, int H, int Skv, int K, int q_start, float sm_scale, const float* __restrict__ sink) {
+    int S, int H, int Skv, int K, int q_start, float sm_scale, const float* __restrict__ sink, int p_skip) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, g = lane >> 5;
@@ -134,10 +134,11 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
   }
 
   // slots of tiles that are never visited still need their -inf in p_out
+  // (p_out holds the slots from p_skip on: its rows are K - p_skip wide)
   if (POUT != 0 && head_ok && ntiles < NT) {
-    for (int t = 0; t < NT; t++) {
+    for (int t = p_skip / BI; t < NT; t++) {
       if (tmask[t] != 0u) continue;
-      const size_t pbase = ((size_t)qi * H + h) * K + (size_t)t * BI + 16 * g;
+      const size_t pbase = ((size_t)qi * H + h) * (K - p_skip) + (size_t)(t * BI - p_skip) + 16 * g;
       if (POUT == 2) {
         const f32x4 ninf = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
@@ -256,8 +257,8 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
 
     f32x16 sacc;
     qk_tile(tb, mask, sacc);
-    if (POUT != 0 && head_ok) {
-      const size_t pbase = ((size_t)qi * H + h) * K + (size_t)tile * BI + 4 * g;
+    if (POUT != 0 && head_ok && tile * BI >= p_skip) {
+      const size_t pbase = ((size_t)qi * H + h) * (K - p_skip) + (size_t)(tile * BI - p_skip) + 4 * g;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         if (POUT == 2) {
@@ -361,7 +362,7 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
 
 template <int STAGES>
 int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K, int q_start,
-               float sm_scale, void* out, float* lse, void* p_out, int p_out_f32, const float* sink, hipStream_t st) {
+               float sm_scale, void* out, float* lse, void* p_out, int p_out_f32, const float* sink, int p_skip, hipStream_t st) {
   const size_t smem = (size_t)STAGES * TILE_BYTES + (size_t)K * 4 + (size_t)(K / BI) * 8 + 16;   // ids, tile masks, tile list, counters
   if (smem > 160 * 1024) return -1;
   dim3 grid(S), block(256);
@@ -370,8 +371,8 @@ int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, 
     auto kern2 = mla_fwd_kernel<STAGES, P, true>; \
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2; \
     if (hipFuncSetAttribute((const void*)kern2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2; \
-    kern<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink); \
-    kern2<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink); \
+    kern<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip); \
+    kern2<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip); \
   } while (0)
   if (!p_out) DSA_FWD_LAUNCH(0);
   else if (!p_out_f32) DSA_FWD_LAUNCH(1);
@@ -382,21 +383,23 @@ int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, 
 
 }  // namespace
 
-extern "C" int dsa_sparse_mla_fwd_sink(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K,
-                                       int q_start, float sm_scale, int d_v, void* out, float* lse, void* p_out,
-                                       int p_out_f32, const float* attn_sink, void* stream) {
+extern "C" int dsa_sparse_mla_fwd_ex(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K,
+                                     int q_start, float sm_scale, int d_v, void* out, float* lse, void* p_out,
+                                     int p_out_f32, const float* attn_sink, int p_out_skip, void* stream) {
   DSA_REQUIRE(d_v == DV, "dsa_sparse_mla_fwd: only d_v = 512 (d_qk = 576) is supported, got d_v = %d", d_v);
   DSA_REQUIRE(S >= 0 && Skv > 0, "dsa_sparse_mla_fwd: bad sequence sizes S=%d Skv=%d", S, Skv);
   DSA_REQUIRE(H > 0 && H <= 128 && H % 32 == 0, "dsa_sparse_mla_fwd: head count must be 32, 64, 96 or 128, got %d", H);
   DSA_REQUIRE(K > 0 && K % 64 == 0, "dsa_sparse_mla_fwd: top-k must be a positive multiple of 64, got %d", K);
+  DSA_REQUIRE(p_out_skip >= 0 && p_out_skip < K && p_out_skip % BI == 0,
+              "dsa_sparse_mla_fwd: p_out_skip must be a multiple of %d in [0, top-k), got %d", BI, p_out_skip);
   DSA_REQUIRE((size_t)Skv * DQK * 2 <= 0xffffffffull, "dsa_sparse_mla_fwd: kv larger than 4 GiB is not supported");
   DSA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)kv % 16) == 0 && ((uintptr_t)out % 8) == 0 &&
               ((uintptr_t)p_out % 16) == 0 && ((uintptr_t)attn_sink % 4) == 0, "dsa_sparse_mla_fwd: misaligned pointer");
   if (S == 0) return DSA_OK;
   hipStream_t st = (hipStream_t)stream;
   int rc;
-  if (K <= 2048) rc = launch_fwd<4>(q, kv, ids, S, H, Skv, K, q_start, sm_scale, out, lse, p_out, p_out_f32, attn_sink, st);
-  else if (K <= 8192) rc = launch_fwd<3>(q, kv, ids, S, H, Skv, K, q_start, sm_scale, out, lse, p_out, p_out_f32, attn_sink, st);
+  if (K <= 2048) rc = launch_fwd<4>(q, kv, ids, S, H, Skv, K, q_start, sm_scale, out, lse, p_out, p_out_f32, attn_sink, p_out ? p_out_skip : 0, st);
+  else if (K <= 8192) rc = launch_fwd<3>(q, kv, ids, S, H, Skv, K, q_start, sm_scale, out, lse, p_out, p_out_f32, attn_sink, p_out ? p_out_skip : 0, st);
   else rc = -1;
   DSA_REQUIRE(rc != -1, "dsa_sparse_mla_fwd: top-k %d exceeds the supported maximum 8192", K);
   if (rc == -2) DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_fwd: cannot reserve LDS");
@@ -407,5 +410,5 @@ extern "C" int dsa_sparse_mla_fwd_sink(const void* q, const void* kv, const int3
 extern "C" int dsa_sparse_mla_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K,
                                   int q_start, float sm_scale, int d_v, void* out, float* lse, void* p_out,
                                   int p_out_f32, void* stream) {
-  return dsa_sparse_mla_fwd_sink(q, kv, ids, S, H, Skv, K, q_start, sm_scale, d_v, out, lse, p_out, p_out_f32, nullptr, stream);
+  return dsa_sparse_mla_fwd_ex(q, kv, ids, S, H, Skv, K, q_start, sm_scale, d_v, out, lse, p_out, p_out_f32, nullptr, 0, stream);
 }

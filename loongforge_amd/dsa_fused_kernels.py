@@ -56,14 +56,20 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
     divisor of it, expanded as at :2040-2046) adds a per-head sink term to the softmax denominator;
     ``topk_length`` ([s_q] int32) keeps only the first ``topk_length[i]`` slots of query ``i``.  No
     gradient is returned for ``attn_sink`` (the reference returns none either, :2112).
-    ``window_size`` belongs to a different attention variant and must keep its default.
+    ``window_size`` (DeepSeek-V4: the leading slots hold the sliding-window keys) leaves those slots
+    out of ``p_out``, which is then [sq, n, topk - window_size]
+    (loongforge/models/foundation/deepseek_v4/deepseek_v4_csa.py:2341-2346); attention runs over every
+    slot.  As in the reference it is only accepted together with ``return_p_out`` (:2971-2974).
     """
 
     @staticmethod
     def forward(ctx, q, kv, indices, chunk_offset=0, sm_scale=None, d_v=512, return_p_out=False,
                 packed_seq_params=None, topk_length=None, attn_sink=None, window_size=0, fast_mode=False):
-        if window_size not in (0, None):
-            raise NotImplementedError("window_size is not supported by this build")
+        window_size = int(window_size or 0)
+        if window_size and not return_p_out:
+            raise ValueError("window_size > 0 needs return_p_out=True")
+        if window_size % 32:
+            raise NotImplementedError("window_size must be a multiple of 32, got %d" % window_size)
         # q [sq, n, d]; kv [skv, 1, d]; indices [sq, 1, topk]
         sq = q.size(0)
         kv2 = kv.reshape(kv.shape[0], kv.shape[-1])
@@ -77,7 +83,7 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
                 attn_sink = attn_sink.flatten().repeat_interleave(h_q // attn_sink.numel())
             attn_sink = attn_sink.contiguous().view(h_q).float()
         out, lse, p_out = ops.sparse_mla_fwd(q, kv2, ids, chunk_offset, sm_scale, d_v, return_p_out,
-                                             attn_sink=attn_sink)
+                                             attn_sink=attn_sink, p_out_skip=window_size)
         ctx.save_for_backward(q, kv, ids, out, lse)
         ctx.sm_scale = sm_scale
         ctx.chunk_offset = chunk_offset

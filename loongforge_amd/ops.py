@@ -278,7 +278,8 @@ def _check_mla(q, kv, ids):
 
 @torch.library.custom_op("dsa::sparse_mla_fwd", mutates_args=())
 def _mla_fwd_op(q: torch.Tensor, kv: torch.Tensor, ids: torch.Tensor, q_start: int, sm_scale: float, d_v: int,
-                p_out_mode: int, attn_sink: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                p_out_mode: int, attn_sink: Optional[torch.Tensor] = None,
+                p_out_skip: int = 0) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     _check_mla(q, kv, ids)
     q, kv, ids = _c(q), _c(kv), _c(ids.int())
     S, H, _ = q.shape
@@ -293,33 +294,39 @@ def _mla_fwd_op(q: torch.Tensor, kv: torch.Tensor, ids: torch.Tensor, q_start: i
     if p_out_mode == 0:
         p_out = torch.empty(0, dtype=torch.bfloat16, device=q.device)
     else:
-        p_out = torch.empty(S, H, K, dtype=torch.float32 if p_out_mode == 2 else torch.bfloat16, device=q.device)
+        if p_out_skip < 0 or p_out_skip >= K or p_out_skip % 32:
+            raise ValueError("p_out_skip must be a multiple of 32 in [0, top-k), got %d" % p_out_skip)
+        p_out = torch.empty(S, H, K - p_out_skip, dtype=torch.float32 if p_out_mode == 2 else torch.bfloat16,
+                            device=q.device)
     lib = _lib.load()
     with torch.cuda.device(q.device):
-        _lib.check(lib.dsa_sparse_mla_fwd_sink(q.data_ptr(), kv.data_ptr(), ids.data_ptr(), S, H, kv.shape[0], K,
-                                               int(q_start), float(sm_scale), int(d_v), out.data_ptr(), lse.data_ptr(),
-                                               p_out.data_ptr() if p_out_mode else None, int(p_out_mode == 2),
-                                               attn_sink.data_ptr() if attn_sink is not None else None, _stream(q)),
+        _lib.check(lib.dsa_sparse_mla_fwd_ex(q.data_ptr(), kv.data_ptr(), ids.data_ptr(), S, H, kv.shape[0], K,
+                                             int(q_start), float(sm_scale), int(d_v), out.data_ptr(), lse.data_ptr(),
+                                             p_out.data_ptr() if p_out_mode else None, int(p_out_mode == 2),
+                                             attn_sink.data_ptr() if attn_sink is not None else None,
+                                             int(p_out_skip), _stream(q)),
                    "dsa_sparse_mla_fwd")
     return out, lse, p_out
 
 
 @_mla_fwd_op.register_fake
-def _(q, kv, ids, q_start, sm_scale, d_v, p_out_mode, attn_sink=None):
+def _(q, kv, ids, q_start, sm_scale, d_v, p_out_mode, attn_sink=None, p_out_skip=0):
     S, H, _ = q.shape
-    p = q.new_empty(0) if p_out_mode == 0 else q.new_empty(S, H, ids.shape[1], dtype=torch.float32 if p_out_mode == 2 else torch.bfloat16)
+    p = q.new_empty(0) if p_out_mode == 0 else q.new_empty(S, H, ids.shape[1] - p_out_skip, dtype=torch.float32 if p_out_mode == 2 else torch.bfloat16)
     return q.new_empty(S, H, d_v), q.new_empty(S, H, dtype=torch.float32), p
 
 
 def sparse_mla_fwd(q, kv, ids, q_start: int = 0, sm_scale: Optional[float] = None, d_v: int = 512,
                    return_p_out: bool = False, p_out_dtype: torch.dtype = torch.bfloat16,
-                   attn_sink: Optional[torch.Tensor] = None):
+                   attn_sink: Optional[torch.Tensor] = None, p_out_skip: int = 0):
     """(out bf16 [S,H,d_v], natural-log lse fp32 [S,H], p_out or None).  ``attn_sink`` [H]: per-head
-    sink logit added to the softmax denominator (and to lse)."""
+    sink logit added to the softmax denominator (and to lse).  ``p_out_skip``: p_out leaves out that
+    many leading slots (a multiple of 32) and is [S,H,K - p_out_skip]."""
     if sm_scale is None:
         sm_scale = q.shape[-1] ** -0.5
     mode = 0 if not return_p_out else (2 if p_out_dtype == torch.float32 else 1)
-    out, lse, p_out = _mla_fwd_op(q, kv, ids, int(q_start), float(sm_scale), int(d_v), mode, attn_sink)
+    out, lse, p_out = _mla_fwd_op(q, kv, ids, int(q_start), float(sm_scale), int(d_v), mode, attn_sink,
+                                   int(p_out_skip) if return_p_out else 0)
     return out, lse, (p_out if return_p_out else None)
 
 

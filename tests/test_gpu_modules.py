@@ -45,7 +45,12 @@ def test_dot_product_attention_layouts_and_autograd(gpu):
     with pytest.raises(AssertionError):
         attn(q.unsqueeze(1), kv.unsqueeze(1), ids.unsqueeze(0), 0, AttnMaskType.no_mask)
     with pytest.raises(NotImplementedError):
-        attn(q.unsqueeze(1), kv.unsqueeze(1), ids.unsqueeze(0), 0, None, window_size=4)
+        attn(q.unsqueeze(1), kv.unsqueeze(1), ids.unsqueeze(0), 0, None, window_size=4, return_p_out=True)
+    with pytest.raises(ValueError):
+        attn(q.unsqueeze(1), kv.unsqueeze(1), ids.unsqueeze(0), 0, None, window_size=64)
+    # window_size: p_out leaves out the leading (window) slots, the output is unchanged
+    out4, p4 = attn(q.unsqueeze(1), kv.unsqueeze(1), ids.unsqueeze(0), 0, None, window_size=64, return_p_out=True)
+    assert p4.shape == (150, 128, 64) and torch.equal(p4, p_out[:, :, 64:]) and torch.equal(out4, out)
     # topk_length keeps a prefix of each query's slots; attn_sink ([h] or a divisor of it) joins the denominator
     tl = torch.randint(0, 101, (150,), generator=torch.Generator().manual_seed(4), dtype=torch.int32)
     sink = torch.linspace(-2, 2, 64)

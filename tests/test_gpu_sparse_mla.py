@@ -50,6 +50,11 @@ def test_forward_p_out_and_attn_dist(gpu):
         ref16 = O.attn_dist(rp[:, :16], inp.sm_scale)
         assert (tgt16.cpu() - ref16).abs().max().item() < (1e-5 if dt == torch.float32 else 6e-3)
         assert triton_attn_dist(p, inp.sm_scale).dtype == dt
+        # leaving out leading slots changes nothing but the width of p_out
+        for skip in (32, 96):
+            o_s, l_s, p_s = ops.sparse_mla_fwd(inp.q.to(gpu), inp.kv.to(gpu), inp.idx.to(gpu), 0, inp.sm_scale, 512, True, dt,
+                                               p_out_skip=skip)
+            assert p_s.shape == (200, 128, 128 - skip) and torch.equal(p_s, p[:, :, skip:])
 
 
 def test_forward_invalid_ids_and_empty_rows(gpu):
