@@ -103,6 +103,15 @@ def main():
     out = torch.empty(S, H, DV, dtype=torch.bfloat16, device=dev)
     lse = torch.empty(S, H, dtype=torch.float32, device=dev)
     pass_ms = (ctypes.c_float * 5)()
+    q8 = torch.empty(S, HI, 128, dtype=torch.uint8, device=dev)
+    k8 = torch.empty(S, 128, dtype=torch.uint8, device=dev)
+    qs = torch.empty(S, HI, dtype=torch.float32, device=dev)
+    ksc = torch.empty(S, dtype=torch.float32, device=dev)
+    wsd = torch.empty(S, HI, dtype=torch.float32, device=dev)
+    sc = torch.empty(S, K, dtype=torch.float32, device=dev)
+    ids = torch.empty(S, K, dtype=torch.int32, device=dev)
+    iwsb = lib.dsa_indexer_topk_workspace_bytes(S, S, K)
+    iws = torch.empty(iwsb, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
 
     def ev():
@@ -118,11 +127,18 @@ def main():
         t0 = time.time()
         e = [ev() for _ in range(6)]
         e[0].record()
-        q8, qs = ops.quant_rowwise_e4m3(iq_d)
-        k8, ksc = ops.quant_rowwise_e4m3(ik_d)
-        wsd = (w_d * qs * 128 ** -0.5).contiguous()
+        # quantise q and k, fold the query scales into the head weights, logits + top-k: straight
+        # through the C ABI on preallocated buffers, like the attention calls below
+        _lib.check(lib.dsa_quant_rowwise_e4m3(iq_d.data_ptr(), S * HI, 128, q8.data_ptr(), qs.data_ptr(), 1e-12, 1,
+                                              stream), "quant q")
+        _lib.check(lib.dsa_quant_rowwise_e4m3(ik_d.data_ptr(), S, 128, k8.data_ptr(), ksc.data_ptr(), 1e-12, 1,
+                                              stream), "quant k")
+        torch.mul(w_d, qs, out=wsd)
+        wsd.mul_(128 ** -0.5)
         e[1].record()
-        sc, ids = ops.indexer_topk(q8, wsd, k8, ksc, ks, ke, K)
+        _lib.check(lib.dsa_indexer_topk_fwd(q8.data_ptr(), wsd.data_ptr(), k8.data_ptr(), ksc.data_ptr(), ks.data_ptr(),
+                                            ke.data_ptr(), S, HI, S, K, 1, sc.data_ptr(), ids.data_ptr(),
+                                            iws.data_ptr(), iwsb, stream), "indexer + top-k")
         e[2].record()
         _lib.check(lib.dsa_sparse_mla_fwd(q.data_ptr(), kv.data_ptr(), idx.data_ptr(), S, H, S, K, 0, inp.sm_scale, DV,
                                           out.data_ptr(), lse.data_ptr(), None, 0, stream), "fwd")

@@ -19,7 +19,9 @@ namespace {
 constexpr int D = 128;          // indexer head dim (bytes per fp8 row)
 constexpr int BK = 128;         // keys per LDS tile
 constexpr int TILE_BYTES = BK * D;
-constexpr int QW = 2;           // queries per wave
+#ifndef IDX_QW
+#define IDX_QW 1                // queries per wave
+#endif
 constexpr int QB = 8;           // queries per workgroup
 
 __device__ __forceinline__ int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
@@ -46,21 +48,34 @@ __global__ void fill_neg_inf_kernel(float* __restrict__ p, long rows, long ld, i
     p[(e / width) * ld + (e % width)] = -INFINITY;
 }
 
-template <int NHT>   // groups of 32 heads
-__global__ __launch_bounds__(256, 2) void indexer_logits_kernel(
+// sum of x over the two half-waves (lanes l and l ^ 32), in every lane.  v_permlane32_swap
+// exchanges the upper half of its first operand with the lower half of its second: afterwards one
+// register holds the lower-half values in both halves and the other the upper-half values.  (Written
+// as inline assembly: given the same value for both operands the compiler's builtin is folded as if
+// both results were equal.)
+__device__ __forceinline__ float add_halves(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+
+template <int NHT, int QW>   // groups of 32 heads; queries per wave (QB / QW waves per workgroup)
+__global__ __launch_bounds__(64 * QB / QW, QW == 1 ? 4 : 2) void indexer_logits_kernel(
     const unsigned char* __restrict__ q8, const float* __restrict__ q_w, const unsigned char* __restrict__ k8,
     const float* __restrict__ k_scale, const int* __restrict__ ks, const int* __restrict__ ke,
     int S, int Sk, float* __restrict__ logits, long ld, int relative, int q_begin, int q_count) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * TILE_BYTES + 2 * BK * 4];
   constexpr int HI = NHT * 32;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int NWAVE = QB / QW;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: window tests below become scalar branches
   const int r = lane & 31, g = lane >> 5;
   const int nblk = (q_count + QB - 1) / QB;
   const int blk = nblk - 1 - (int)blockIdx.x;            // longest windows first
   const int qb0 = q_begin + blk * QB;
   const int q_end = q_begin + q_count;
 
-  // window union of the block (wave-uniform scalars)
+  // window union of the block
   int jlo = 0x7fffffff, jhi = 0;
   for (int t = 0; t < QB; t++) {
     const int i = qb0 + t;
@@ -70,6 +85,7 @@ __global__ __launch_bounds__(256, 2) void indexer_logits_kernel(
 
   // this wave's queries
   int qi[QW], qks[QW], qke[QW];
+  int wlo = 0x7fffffff, whi = 0;                         // union of the wave's windows
   i32x8 aq[QW][NHT][2];
   float wq[QW][NHT][16];
 #pragma unroll
@@ -79,6 +95,7 @@ __global__ __launch_bounds__(256, 2) void indexer_logits_kernel(
     qi[u] = live ? i : -1;
     qks[u] = live ? max(ks[i], 0) : 0;
     qke[u] = live ? min(ke[i], Sk) : 0;
+    if (live) { wlo = min(wlo, qks[u]); whi = max(whi, qke[u]); }
     const int is = live ? i : qb0;
 #pragma unroll
     for (int t = 0; t < NHT; t++) {
@@ -108,17 +125,17 @@ __global__ __launch_bounds__(256, 2) void indexer_logits_kernel(
 
   const int t_lo = jlo / BK, t_hi = (jhi + BK - 1) / BK;      // key tiles [t_lo, t_hi)
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
-  const int gkey = tid >> 3, gsub = tid & 7;                  // 32 key rows per DMA instruction
+  const int gkey = tid >> 3, gsub = tid & 7;                  // 8 NWAVE key rows per DMA instruction
   auto issue = [&](int t) {
-    const unsigned lb = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)((t & 1) * TILE_BYTES + wave * 1024));
+    const unsigned lb = lds0 + (unsigned)((t & 1) * TILE_BYTES + wave * 1024);
 #pragma unroll
-    for (int c = 0; c < BK / 32; c++) {
-      const int key = c * 32 + gkey;
+    for (int c = 0; c < BK / (8 * NWAVE); c++) {
+      const int key = c * 8 * NWAVE + gkey;
       const int row = min(t * BK + key, Sk - 1);
-      dma16(lb + c * 4096, (unsigned)row * D + (unsigned)((gsub ^ swz(key)) * 16), k8);
+      dma16(lb + c * 1024 * NWAVE, (unsigned)row * D + (unsigned)((gsub ^ swz(key)) * 16), k8);
     }
     if (wave < BK / 64) {   // the tile's per-key scales
-      const unsigned sb = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(2 * TILE_BYTES + (t & 1) * BK * 4 + wave * 256));
+      const unsigned sb = lds0 + (unsigned)(2 * TILE_BYTES + (t & 1) * BK * 4 + wave * 256);
       dma4(sb, (unsigned)min(t * BK + wave * 64 + lane, Sk - 1) * 4u, k_scale);
     }
   };
@@ -139,7 +156,7 @@ __global__ __launch_bounds__(256, 2) void indexer_logits_kernel(
 #pragma unroll 1
     for (int c = 0; c < BK / 32; c++) {
       const int j0 = t * BK + c * 32;
-      if (j0 >= jhi) break;
+      if (j0 >= whi || j0 + 32 <= wlo) continue;               // scalar: nothing of this wave's windows here
       const int j = j0 + r;
       const unsigned char* cb = tb + c * 32 * D;
       i32x8 bk[2];
@@ -152,28 +169,22 @@ __global__ __launch_bounds__(256, 2) void indexer_logits_kernel(
       const float ksc = ksc_s[c * 32 + r];
 #pragma unroll
       for (int u = 0; u < QW; u++) {
-        if (qi[u] < 0) continue;
-        const bool any = (j0 < qke[u]) && (j0 + 32 > qks[u]);     // wave-uniform
+        if (QW > 1 && (qi[u] < 0 || j0 >= qke[u] || j0 + 32 <= qks[u])) continue;   // scalar
         float part = 0.f;
-        if (any) {
 #pragma unroll
-          for (int tt = 0; tt < NHT; tt++) {
-            f32x16 acc;
+        for (int tt = 0; tt < NHT; tt++) {
+          f32x16 acc;
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[e] = 0.f;
-            acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[u][tt][0], bk[0], acc, 0, 0, 0, 127, 0, 127);
-            acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[u][tt][1], bk[1], acc, 0, 0, 0, 127, 0, 127);
+          for (int e = 0; e < 16; e++) acc[e] = 0.f;
+          acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[u][tt][0], bk[0], acc, 0, 0, 0, 127, 0, 127);
+          acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[u][tt][1], bk[1], acc, 0, 0, 0, 127, 0, 127);
 #pragma unroll
-            for (int e = 0; e < 16; e++) part = fmaf(wq[u][tt][e], relu1(acc[e]), part);
-          }
-          part += __shfl_xor(part, 32, 64);
-          part *= ksc;
+          for (int e = 0; e < 16; e++) part = fmaf(wq[u][tt][e], relu1(acc[e]), part);
         }
-        if (g == 0) {
-          const bool vis = any && j >= qks[u] && j < qke[u];
+        part = add_halves(part) * ksc;
+        if (g == 0 && j >= qks[u] && j < qke[u]) {
           const int col = relative ? j - qks[u] : j;
-          float* dst = logits + (size_t)(qi[u] - q_begin) * ld;
-          if (vis) dst[col] = part;
+          logits[(size_t)(qi[u] - q_begin) * ld + col] = part;
         }
       }
     }
@@ -198,8 +209,9 @@ int dsa_indexer_logits_block(const void* q8, const float* q_w, const void* k8, c
     fill_neg_inf_kernel<<<dim3(2048), dim3(256), 0, st>>>(logits, q_count, (long)ld, width);
     DSA_CHECK_LAUNCH("dsa_indexer_logits(fill)");
   }
-  dim3 grid((q_count + QB - 1) / QB), block(256);
-#define DSA_IDX_LAUNCH(N) indexer_logits_kernel<N><<<grid, block, 0, st>>>( \
+  constexpr int QW = IDX_QW;
+  dim3 grid((q_count + QB - 1) / QB), block(64 * QB / QW);
+#define DSA_IDX_LAUNCH(N) indexer_logits_kernel<N, QW><<<grid, block, 0, st>>>( \
     (const unsigned char*)q8, q_w, (const unsigned char*)k8, k_scale, ks, ke, S, Sk, logits, (long)ld, relative, q_begin, q_count)
   if (Hi == 32) DSA_IDX_LAUNCH(1);
   else DSA_IDX_LAUNCH(2);

@@ -146,8 +146,73 @@ __device__ __forceinline__ void bitonic_regs(float* outv, int* outi, unsigned lo
 // of the threshold bin that rank beyond the K-th place are dropped.  The result is exact and does
 // not depend on the order in which the atomics land.  Returns false without writing anything when
 // the row is unsuitable (no spread, or a crowded bin): the caller then takes the general path.
-constexpr int LIN_SPARE = 1024;              // extra buffer entries for the threshold bin's surplus
+constexpr int LIN_SPARE = 960;               // extra buffer entries for the threshold bin's surplus
+constexpr int REG_ROW = 8192 + 4 * 256;      // longest row (plus alignment slack) the register variant holds
 constexpr int LIN_MAX_BIN = 256;             // largest segment ranked by pairwise counting
+
+// Threshold bin of a filled histogram (thread t owns bins [PER t, PER t + PER)), then the segment
+// starts written over the counts.  False when a bin is too crowded for the ranking step.
+__device__ __forceinline__ bool lin_threshold(int* hist, int* scratch, int keff, int& tbin, int& above, int& c) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int PER = HBINS / BLOCK;
+  int cnt[PER], local = 0;
+#pragma unroll
+  for (int b4 = 0; b4 < PER; b4 += 4) {
+    const int4 q4 = *(const int4*)(hist + tid * PER + b4);
+    cnt[b4] = q4.x; cnt[b4 + 1] = q4.y; cnt[b4 + 2] = q4.z; cnt[b4 + 3] = q4.w;
+  }
+#pragma unroll
+  for (int b = 0; b < PER; b++) local += cnt[b];
+  int total;
+  const int before = block_exscan(local, scratch, total);
+  if (before < keff && before + local >= keff) {
+    int run = before;
+#pragma unroll
+    for (int b = 0; b < PER; b++) {
+      if (run < keff && run + cnt[b] >= keff) { scratch[8] = tid * PER + b; scratch[9] = run; scratch[10] = cnt[b]; }
+      run += cnt[b];
+    }
+  }
+  __syncthreads();
+  tbin = scratch[8]; above = scratch[9]; c = scratch[10];
+  int big = 0;
+#pragma unroll
+  for (int b = 0; b < PER; b++) if (tid * PER + b < tbin) big = max(big, cnt[b]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) big = max(big, __shfl_xor(big, o, 64));
+  __syncthreads();
+  if (lane == 0) scratch[wave] = big;
+  __syncthreads();
+  big = max(max(scratch[0], scratch[1]), max(scratch[2], scratch[3]));
+  if (big > LIN_MAX_BIN || c > LIN_SPARE) return false;
+  {
+    int run = before, st[PER];
+#pragma unroll
+    for (int b = 0; b < PER; b++) { st[b] = run; run += cnt[b]; }
+#pragma unroll
+    for (int b4 = 0; b4 < PER; b4 += 4) *(int4*)(hist + tid * PER + b4) = make_int4(st[b4], st[b4 + 1], st[b4 + 2], st[b4 + 3]);
+  }
+  __syncthreads();
+  return true;
+}
+
+// Final position of every scattered element: hist[b] is the end of segment b by now.
+template <class BinOf>
+__device__ __forceinline__ void lin_rank(const unsigned long long* obuf, const int* hist, int filled, int keff, int K,
+                                         int base_id, BinOf bin_of, float* sv, int* si) {
+  const int tid = threadIdx.x;
+  for (int p = tid; p < filled; p += BLOCK) {
+    const unsigned long long key = obuf[p];
+    const float v = sort_key_score(key);
+    const int b = bin_of(v);
+    const int start = b > 0 ? hist[b - 1] : 0, end = hist[b];
+    int rank = 0;
+    for (int j = start; j < end; j++) rank += obuf[j] < key;
+    const int pos = start + rank;
+    if (pos < keff) { sv[pos] = v; si[pos] = base_id + (int)(unsigned)key; }
+  }
+  for (int t = keff + tid; t < K; t += BLOCK) { sv[t] = -INFINITY; si[t] = -1; }
+}
 
 __device__ __forceinline__ bool linear_select_sort(const float* __restrict__ src, unsigned* keys, int n, int K, int base_id,
                                                    int* hist, int* scratch, unsigned long long* obuf, float* sv, int* si) {
@@ -191,47 +256,9 @@ __device__ __forceinline__ bool linear_select_sort(const float* __restrict__ src
     if (fabsf(v) < INFINITY) atomicAdd(&hist[bin_of(v)], 1);
   }
   __syncthreads();
-  // ---- threshold bin: thread t owns bins [16t, 16t + 16) -------------------------------------------
-  constexpr int PER = HBINS / BLOCK;
-  int cnt[PER], local = 0;
-#pragma unroll
-  for (int b4 = 0; b4 < PER; b4 += 4) {
-    const int4 q4 = *(const int4*)(hist + tid * PER + b4);
-    cnt[b4] = q4.x; cnt[b4 + 1] = q4.y; cnt[b4 + 2] = q4.z; cnt[b4 + 3] = q4.w;
-  }
-#pragma unroll
-  for (int b = 0; b < PER; b++) local += cnt[b];
-  int total;
-  const int before = block_exscan(local, scratch, total);
-  if (before < keff && before + local >= keff) {
-    int run = before;
-#pragma unroll
-    for (int b = 0; b < PER; b++) {
-      if (run < keff && run + cnt[b] >= keff) { scratch[8] = tid * PER + b; scratch[9] = run; scratch[10] = cnt[b]; }
-      run += cnt[b];
-    }
-  }
-  __syncthreads();
-  const int tbin = scratch[8], above = scratch[9], c = scratch[10];
-  int big = 0;
-#pragma unroll
-  for (int b = 0; b < PER; b++) if (tid * PER + b < tbin) big = max(big, cnt[b]);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) big = max(big, __shfl_xor(big, o, 64));
-  __syncthreads();
-  if (lane == 0) scratch[wave] = big;
-  __syncthreads();
-  big = max(max(scratch[0], scratch[1]), max(scratch[2], scratch[3]));
-  if (big > LIN_MAX_BIN || c > LIN_SPARE) return false;
-  // ---- segment starts (in place), scatter -------------------------------------------------------
-  {
-    int run = before, st[PER];
-#pragma unroll
-    for (int b = 0; b < PER; b++) { st[b] = run; run += cnt[b]; }
-#pragma unroll
-    for (int b4 = 0; b4 < PER; b4 += 4) *(int4*)(hist + tid * PER + b4) = make_int4(st[b4], st[b4 + 1], st[b4 + 2], st[b4 + 3]);
-  }
-  __syncthreads();
+  int tbin, above, c;
+  if (!lin_threshold(hist, scratch, keff, tbin, above, c)) return false;
+  // ---- scatter ------------------------------------------------------------------------------------
   for (int e = tid; e < n; e += BLOCK) {
     const float v = key2f(keys[e]);
     if (fabsf(v) < INFINITY) {
@@ -240,24 +267,84 @@ __device__ __forceinline__ bool linear_select_sort(const float* __restrict__ src
     }
   }
   __syncthreads();
-  // ---- rank inside the segment: hist[b] is now the end of segment b ------------------------------
-  const int filled = above + c;
-  for (int p = tid; p < filled; p += BLOCK) {
-    const unsigned long long key = obuf[p];
-    const float v = sort_key_score(key);
-    const int b = bin_of(v);
-    const int start = b > 0 ? hist[b - 1] : 0, end = hist[b];
-    int rank = 0;
-    for (int j = start; j < end; j++) rank += obuf[j] < key;
-    const int pos = start + rank;
-    if (pos < keff) { sv[pos] = v; si[pos] = base_id + (int)(unsigned)key; }
-  }
-  for (int t = keff + tid; t < K; t += BLOCK) { sv[t] = -INFINITY; si[t] = -1; }
+  lin_rank(obuf, hist, above + c, keff, K, base_id, bin_of, sv, si);
   return true;
 }
 
-template <bool STAGED>
-__global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ logits, long ld,
+// The same for rows of at most 4 NV BLOCK elements, with the row held in registers instead of
+// LDS: thread t owns the 16-byte chunks t, t + BLOCK, ... of the row counted from the 16-byte
+// boundary at or below its first element, so the whole row is fetched by NV vector loads issued
+// together and the workgroup needs only the histogram and the output buffer in LDS.
+template <int NV>
+__device__ __forceinline__ bool linear_select_sort_regs(const float* __restrict__ src, int n, int K, int base_id,
+                                                        int* hist, int* scratch, unsigned long long* obuf, float* sv, int* si) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int off = (int)(((uintptr_t)src >> 2) & 3);        // elements between that boundary and src
+  const float* base = src - off;
+  const int m = n + off;                                    // the row is [off, m) of base
+  float v[NV][4];
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int p = 4 * (tid + BLOCK * i);
+    if (p >= off && p + 4 <= m) {
+      const float4 x = *(const float4*)(base + p);
+      v[i][0] = x.x; v[i][1] = x.y; v[i][2] = x.z; v[i][3] = x.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[i][j] = (p + j >= off && p + j < m) ? base[p + j] : -INFINITY;
+    }
+  }
+  for (int b = tid; b < HBINS; b += BLOCK) hist[b] = 0;
+  float mn = INFINITY, mx = -INFINITY;
+  int nfin = 0;
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (fabsf(v[i][j]) < INFINITY) { mn = fminf(mn, v[i][j]); mx = fmaxf(mx, v[i][j]); nfin++; }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    nfin += __shfl_xor(nfin, o, 64);
+  }
+  if (lane == 0) { ((float*)scratch)[wave] = mn; ((float*)scratch)[4 + wave] = mx; scratch[8 + wave] = nfin; }
+  __syncthreads();
+  mn = fminf(fminf(((float*)scratch)[0], ((float*)scratch)[1]), fminf(((float*)scratch)[2], ((float*)scratch)[3]));
+  mx = fmaxf(fmaxf(((float*)scratch)[4], ((float*)scratch)[5]), fmaxf(((float*)scratch)[6], ((float*)scratch)[7]));
+  nfin = scratch[8] + scratch[9] + scratch[10] + scratch[11];
+  __syncthreads();
+  const float span = mx - mn;
+  if (!(span > 0.f) || !(span < INFINITY)) return false;
+  const int keff = min(K, nfin);
+  const float scale = ((float)HBINS - 0.5f) / span;
+  auto bin_of = [&](float x) { return min(HBINS - 1, (int)((mx - x) * scale)); };
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (fabsf(v[i][j]) < INFINITY) atomicAdd(&hist[bin_of(v[i][j])], 1);
+  __syncthreads();
+  int tbin, above, c;
+  if (!lin_threshold(hist, scratch, keff, tbin, above, c)) return false;
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (fabsf(v[i][j]) < INFINITY) {
+        const int b = bin_of(v[i][j]);
+        if (b <= tbin) obuf[atomicAdd(&hist[b], 1)] = sort_key(v[i][j], 4 * (tid + BLOCK * i) + j - off);
+      }
+  __syncthreads();
+  lin_rank(obuf, hist, above + c, keff, K, base_id, bin_of, sv, si);
+  return true;
+}
+
+// LEAN (sorted rows that fit the register variant; implies !STAGED): the kernel keeps to 128
+// registers so that four workgroups share a compute unit; rows the single-sweep path turns down
+// take the general path on global memory and the plain LDS sorting network.
+template <bool STAGED, bool LEAN>
+__global__ __launch_bounds__(BLOCK, LEAN ? 4 : 1) void topk_kernel(const float* __restrict__ logits, long ld,
                                                      const int* __restrict__ row_begin, const int* __restrict__ row_end,
                                                      int width, const int* __restrict__ id_base, int K, int Kp2, int sorted,
                                                      float* __restrict__ scores, int* __restrict__ ids, int nmax) {
@@ -280,9 +367,19 @@ __global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ l
 
   auto key_at = [&](int e) -> unsigned { return STAGED ? keys[e] : f2key(src[e]); };
 
-  if (STAGED && sorted && n > 0) {   // single-sweep path, also for rows shorter than K
-    if (linear_select_sort(src, keys, n, K, base_id, hist, scratch, (unsigned long long*)outv, sv, si)) return;
-    __syncthreads();
+  if (sorted && n > 0) {   // single-sweep path, also for rows shorter than K
+    if (STAGED) {
+      if (linear_select_sort(src, keys, n, K, base_id, hist, scratch, (unsigned long long*)outv, sv, si)) return;
+      __syncthreads();
+    } else if (LEAN && n + 3 <= REG_ROW) {
+      bool done;
+      unsigned long long* obuf = (unsigned long long*)outv;
+      if (n + 3 <= 8 * BLOCK) done = linear_select_sort_regs<2>(src, n, K, base_id, hist, scratch, obuf, sv, si);
+      else if (n + 3 <= 16 * BLOCK) done = linear_select_sort_regs<4>(src, n, K, base_id, hist, scratch, obuf, sv, si);
+      else done = linear_select_sort_regs<REG_ROW / (4 * BLOCK)>(src, n, K, base_id, hist, scratch, obuf, sv, si);
+      if (done) return;
+      __syncthreads();
+    }
   }
   if (n <= K) {
     for (int t = tid; t < Kp2; t += BLOCK) {
@@ -349,7 +446,7 @@ __global__ __launch_bounds__(BLOCK) void topk_kernel(const float* __restrict__ l
   __syncthreads();
 
   if (sorted) {   // bitonic sort, descending score, ascending id among equal scores
-    const int ept = Kp2 / BLOCK;
+    const int ept = LEAN ? 0 : Kp2 / BLOCK;
     if (ept == 8) { bitonic_regs<8>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
     else if (ept == 4) { bitonic_regs<4>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
     else if (ept == 2) { bitonic_regs<2>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
@@ -387,9 +484,11 @@ int dsa_topk_launch(const float* logits, int S, int64_t ld, const int32_t* row_b
   while (Kp2 < K) Kp2 <<= 1;
   const size_t fixed = (size_t)HBINS * 4 + 64 + (size_t)Kp2 * 8 + (size_t)LIN_SPARE * 8;
   const size_t staged = fixed + (size_t)width * 4;
-  const bool use_staged = staged <= 160 * 1024;
+  // sorted rows that fit the register variant need no staging buffer: four workgroups share a compute unit
+  const bool lean = sorted && width + 3 <= REG_ROW;
+  const bool use_staged = !lean && staged <= 160 * 1024;
   const size_t smem = use_staged ? staged : fixed;
-  auto kern = use_staged ? topk_kernel<true> : topk_kernel<false>;
+  auto kern = lean ? topk_kernel<false, true> : use_staged ? topk_kernel<true, false> : topk_kernel<false, false>;
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
     DSA_FAIL(DSA_ERR_LAUNCH, "dsa_topk: cannot reserve %zu bytes of LDS", smem);
   kern<<<dim3(S), dim3(BLOCK), smem, st>>>(logits, (long)ld, row_begin, row_end, width, id_base, K, Kp2, sorted,

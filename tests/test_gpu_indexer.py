@@ -152,7 +152,7 @@ def test_topk_rule_on_crafted_rows(gpu, kind, K, sorted_out):
     expectation is a stable sort by the library routine."""
     from loongforge_amd import ops
 
-    n, rows = 6000, 12
+    n, rows = 6001, 12                                    # odd width: row starts at every 4-byte alignment
     g = torch.Generator().manual_seed(5)
     x = torch.randn(rows, n, generator=g)
     if kind == "ties":
@@ -169,11 +169,12 @@ def test_topk_rule_on_crafted_rows(gpu, kind, K, sorted_out):
     end = torch.full((rows,), n, dtype=torch.int32)
     if kind == "short":
         end = torch.tensor([1, 2, 63, 64, 255, 256, 257, 999, 1000, 1001, 2047, 2049], dtype=torch.int32)
-    beg = torch.zeros(rows, dtype=torch.int32)
+    beg = torch.zeros(rows, dtype=torch.int32) if kind == "short" else (torch.arange(rows, dtype=torch.int32) % 5)
     sc, ids = ops.topk(x.to(gpu), K, beg.to(gpu), end.to(gpu), sorted=sorted_out)
     sc, ids = sc.cpu(), ids.cpu()
     for i in range(rows):
-        row = x[i, : int(end[i])]
+        row = x[i, : int(end[i])].clone()
+        row[: int(beg[i])] = float("-inf")                  # columns before the window cannot be selected
         order = torch.sort(-row, stable=True).indices      # descending value, ascending column among equals
         fin = torch.isfinite(row[order])
         exp_ids = order[fin][:K]
@@ -186,6 +187,22 @@ def test_topk_rule_on_crafted_rows(gpu, kind, K, sorted_out):
             assert torch.equal(torch.sort(got).values, torch.sort(exp_ids).values), (kind, K, i)
             assert torch.equal(sc[i][ids[i] >= 0], row[got])
         assert (ids[i, kk:] == -1).all() and torch.isinf(sc[i, kk:]).all() and (sc[i, kk:] < 0).all()
+
+
+def test_topk_on_full_width_rows_at_every_alignment(gpu):
+    """Rows of the widest size the register-resident path takes (8192), starting 0..3 elements past a
+    16-byte boundary."""
+    from loongforge_amd import ops
+
+    g = torch.Generator().manual_seed(11)
+    buf = torch.randn(4 * 8192 + 3, generator=g).to(gpu)
+    for off in range(4):
+        x = buf[off: off + 4 * 8192].view(4, 8192)
+        assert x.data_ptr() % 16 == 4 * off
+        sc, ids = ops.topk(x, 2048)
+        ref = torch.sort(-x.cpu(), stable=True, dim=-1).indices[:, :2048]
+        assert torch.equal(ids.cpu().long(), ref)
+        assert torch.equal(sc.cpu(), torch.gather(x.cpu(), 1, ref))
 
 
 def test_fused_rotation_and_quantiser(gpu):
