@@ -160,6 +160,9 @@ def main():
     t_idx, t_fwd, t_bwd = t_idx / n, t_fwd / n, t_bwd / n
     t_pass = [x / n for x in t_pass]
     # separate timing of the two indexer kernels (logits with dense layout + top-k on it)
+    lg = ops.indexer_logits(q8, wsd, k8, ksc, ks, ke)          # untimed first call
+    ops.topk(lg, K, ks, ke)
+    torch.cuda.synchronize()
     e0, e1, e2 = ev(), ev(), ev()
     e0.record()
     lg = ops.indexer_logits(q8, wsd, k8, ksc, ks, ke)
