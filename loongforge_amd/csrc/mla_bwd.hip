@@ -214,8 +214,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
 
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
   const LaneOffsets lo = lane_offsets();
-  // transposed read of the dS block [head group][s'][g'][key][8 heads]: lane (blk, ii) points at
-  // key 16s + 8t + 4g + ii/4 and the 4 heads 16*(blk&1) + 4*(ii&3) .. +3 of a head group
+  // transposed read of the dS block: lane (blk, ii) points at key 16s + 8t + 4g + ii/4 and the 4 heads
+  // 16*(blk&1) + 4*(ii&3) .. +3 of a head group.  In HBM the block is [head group][s'][g'][key][8 heads];
+  // in LDS the 16-byte pieces of a head group are reordered to [key][s'][g'], so that the 16 pieces a
+  // half-wave reads at once (4 keys x 4 head octets) are 256 consecutive bytes: no bank conflicts.
   unsigned ds_off[2][2];
   {
     const int blk = lane >> 4, ii = lane & 15, qq = ii & 3;
@@ -224,9 +226,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         const int key = 16 * s + 8 * t + 4 * g + (ii >> 2);
-        ds_off[s][t] = (unsigned)(TILE_BYTES + (blk & 1) * 1024 + (qq & 1) * 512 + key * 16 + (qq >> 1) * 8);
+        ds_off[s][t] = (unsigned)(TILE_BYTES + key * 64 + (blk & 1) * 32 + (qq & 1) * 16 + (qq >> 1) * 8);
       }
   }
+  // piece P of the LDS order comes from piece src_piece(P) of the HBM order
+  auto src_piece = [](int P) { return (P >> 7) * 128 + ((P >> 1) & 1) * 64 + (P & 1) * 32 + ((P >> 2) & 31); };
+  const unsigned ds_src0 = (unsigned)src_piece(tid) * 16u, ds_src1 = (unsigned)src_piece(tid + 256) * 16u;
   // key-tile operand offsets of this wave's d-tiles: i = 0..3 -> d-tile 4*wave + i, i = 4 -> 16 + wave/2
   const unsigned grp_main = (unsigned)(2 * wave) * GRP_BYTES;          // (4w + i) >> 1 = 2w + (i >> 1)
   const unsigned grp_last = (unsigned)(8 * GRP_BYTES);                 // (16 + w/2) >> 1 = 8
@@ -251,8 +256,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
     gather_tile(kv, idx_s, tile, sb);
     const unsigned lb = __builtin_amdgcn_readfirstlane(sb + (unsigned)(TILE_BYTES + wave * 1024));
     const unsigned char* src = uniform_ptr(pds + ((size_t)ql * NT + tile) * PDS_TILE_BYTES);     // dS half
-    dma16(lb, (unsigned)(tid * 16), src);
-    dma16(lb + 4096, (unsigned)(4096 + tid * 16), src);
+    dma16(lb, ds_src0, src);
+    dma16(lb + 4096, ds_src1, src);
   };
 
   f32x16 acc[18];     // u < 16: d-tile 4*wave + u/4, head group u%4; u = 16, 17: d-tile 16 + wave/2, head group hg_last + u - 16
