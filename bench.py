@@ -171,6 +171,34 @@ def main():
     e2.record()
     torch.cuda.synchronize()
     t_logits, t_topk = e0.elapsed_time(e1), e1.elapsed_time(e2)
+    # one forward with cold caches (a 1 GiB fill evicts L2 and the memory-side cache first)
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    flush.fill_(1)
+    e0, e1 = ev(), ev()
+    e0.record()
+    _lib.check(lib.dsa_sparse_mla_fwd(q.data_ptr(), kv.data_ptr(), idx.data_ptr(), S, H, S, K, 0, inp.sm_scale, DV,
+                                      out.data_ptr(), lse.data_ptr(), None, 0, stream), "fwd")
+    e1.record()
+    torch.cuda.synchronize()
+    t_fwd_cold = e0.elapsed_time(e1)
+    del flush
+    # neighbouring step of the path: q_content permute + rotary embedding + concatenation at the same shape
+    from loongforge_amd.dsa_fused_kernels import fused_rope_permute_cat
+    qc = torch.empty(H, S, DV, dtype=torch.bfloat16, device=dev).normal_()
+    qpe = torch.empty(S, 1, H, DQK - DV, dtype=torch.bfloat16, device=dev).normal_()
+    ang = torch.arange(S, device=dev, dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(0, 64, 2, device=dev) / 64.0))
+    cos_t = torch.cat([ang.cos(), ang.cos()], -1).view(S, 1, 1, 64).contiguous()
+    sin_t = torch.cat([ang.sin(), ang.sin()], -1).view(S, 1, 1, 64).contiguous()
+    fused_rope_permute_cat(qc, qpe, cos_t, sin_t)
+    torch.cuda.synchronize()
+    e0, e1 = ev(), ev()
+    e0.record()
+    for _ in range(5):
+        fused_rope_permute_cat(qc, qpe, cos_t, sin_t)
+    e1.record()
+    torch.cuda.synchronize()
+    t_rope = e0.elapsed_time(e1) / 5
+    del qc, qpe
 
     mla_tflops = (flops_fwd + flops_bwd) / ((t_fwd + t_bwd) * 1e-3) / 1e12
     # ---- roofline of the longest-running kernel of the step ---------------------------------------
@@ -238,6 +266,13 @@ def main():
         "indexer_topk_frac_of_fp8_peak": round(flops_idx / (t_idx * 1e-3) / 1e12 / PEAK_FP8, 4),
         "indexer_logits_ms": round(t_logits, 3), "topk_ms": round(t_topk, 3),
         "topk_hbm_gbps": round((4.0 * vis + 8.0 * S * K) / (t_topk * 1e-3) / 1e9, 1),
+        "mla_fwd_ms_cold_caches": round(t_fwd_cold, 3),
+        "mla_fwd_gather_gbps": round(2.0 * DQK * pairs / (t_fwd * 1e-3) / 1e9, 1),
+        "nominal": {"note": "the same times priced on S*K pairs and S*S logits, as the reference's own print-outs do",
+                    "mla_fwd_bwd_tflops": round(2.0 * H * (4 * DQK + 3 * DV) * S * K / ((t_fwd + t_bwd) * 1e-3) / 1e12, 1),
+                    "indexer_topk_fp8_tflops": round(2.0 * HI * 128 * S * S / (t_idx * 1e-3) / 1e12, 1)},
+        "rope_permute_cat_ms": round(t_rope, 3),
+        "rope_permute_cat_gbps": round(4.0 * S * H * DQK / (t_rope * 1e-3) / 1e9, 1),
         "wall_s_per_step": round(wall / n, 4),
         "roofline": roofline,
     }

@@ -177,6 +177,48 @@ int dsa_sparse_mla_bwd_profile(const void* q, const void* kv, const void* out, c
 int dsa_attn_dist(const void* p_out, int p_out_f32, int S, int H, int K, int64_t ld_s,
                   int64_t ld_h, float sm_scale, float* target, void* stream);
 
+/*
+ * Rotary position embedding of the MLA query / key rows, fused with the copies around it.  Per
+ * (token, head) the call copies a "main" part of d_main bf16 elements between two strided tensors
+ * (main_src NULL: no main part) and rotates a "pe" part of emb_dim bf16 elements, pair by pair:
+ *     y1 = x1 * c1 - x2 * s1     y2 = x2 * c2 + x1 * s2          (inverse = 0)
+ *     y1 = x1 * c1 + x2 * s2     y2 = x2 * c2 - x1 * s1          (inverse = 1: the transpose, for gradients)
+ * in fp32 without fused multiply-adds, rounded once to bf16.  A pairing says where pair i sits in
+ * a row: 0 = adjacent (elements 2i, 2i+1), 1 = split (elements i, i + emb_dim/2); in_pairing and
+ * out_pairing are independent, and cos / sin ([positions, emb_dim], fp32 or bf16) are indexed
+ * with the pairing of the rotated side (out_pairing when inverse = 0, in_pairing when inverse = 1).
+ * Strides are in elements; a pe head stride of 0 broadcasts one row to every head; pe_src may
+ * equal pe_dst when the pairings are equal (in place).  The position of token t is positions[t],
+ * or t / batch when positions is NULL.  Rows must start on 16-byte boundaries, d_main and emb_dim
+ * are multiples of 8.
+ *
+ * This one entry point replaces the reference's Triton kernels
+ *   rotary_{fwd,bwd}_q_kernel_interleaved            dsa_fused_kernels.py:68-228    (in = out = 0, no main part, in place)
+ *   rotary_{fwd,bwd}_q_kernel_non_interleaved        dsa_fused_kernels.py:366-499   (in = out = 1, no main part, in place)
+ *   fused_rope_permute_cat_{fwd,bwd}_kernel_*        dsa_fused_kernels.py:619-1008  (main: [h,S,d] <-> [S,h,d]; in 0 -> out 1 or 0)
+ *   rotary_fwd_absorb_kv_kernel_*                    dsa_fused_kernels.py:1228-1502 (pe head stride 0; in 0 -> out 1 or 0)
+ * and, with emb_dim = 0 (main part only), the k_dim copy of rotary_bwd_absorb_kv_kernel_* (:1327-1371,
+ * :1517-1562); dsa_rope_headsum_inverse is the rest of that kernel.
+ */
+int dsa_rope_rows(const void* main_src, int64_t ms_tok, int64_t ms_head, void* main_dst, int64_t md_tok,
+                  int64_t md_head, int d_main, const void* pe_src, int64_t ps_tok, int64_t ps_head,
+                  void* pe_dst, int64_t pd_tok, int64_t pd_head, int emb_dim, const void* cos,
+                  const void* sin, int cos_sin_f32, const int32_t* positions, int batch, int tokens,
+                  int heads, int in_pairing, int out_pairing, int inverse, void* stream);
+
+/*
+ * Gradient of a pe row that the forward broadcast to every head (the key's rotary part):
+ *   d_emb[t, :] = inverse rotation of bf16( sum_h grad[t, h, :] )   written with adjacent pairing,
+ * the head-sum in fp32 in a fixed order.  grad points at the pe part of the incoming gradient
+ * (element strides g_tok, g_head), in_pairing is the pairing the forward wrote it with.
+ * Replaces the `pid_head == 0` branch of rotary_bwd_absorb_kv_kernel_{non_interleaved,interleaved},
+ * dsa_fused_kernels.py:1372-1410 and :1563-1608.
+ */
+int dsa_rope_headsum_inverse(const void* grad, int64_t g_tok, int64_t g_head, void* d_emb, int64_t de_tok,
+                             int emb_dim, const void* cos, const void* sin, int cos_sin_f32,
+                             const int32_t* positions, int batch, int tokens, int heads, int in_pairing,
+                             void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -292,3 +292,193 @@ class DSAIndexerKernel(torch.nn.Module):
     def forward(self, index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params, rotate=False):
         return DSAIndexerKernelFunction.apply(index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params,
                                               rotate)
+
+
+# ---------------------------------------------------------------------------------------------------
+# MLA rotary embedding fused with permute / concatenate (reference: Triton kernels at
+# dsa_fused_kernels.py:54-1841; here one HIP kernel parameterised by where a rotation pair sits)
+# ---------------------------------------------------------------------------------------------------
+def _token_positions(cu_seqlens, tokens, cp_rank, cp_size, offset=0):
+    """None for sbhd (position = row // batch); for thd the position of each packed token in its own
+    sequence (what megatron's ``_get_thd_token_idx`` returns for context-parallel size 1)."""
+    if cu_seqlens is None:
+        return None
+    if cp_size not in (None, 1):
+        raise NotImplementedError("context parallelism is not supported by this single-GPU build")
+    return ops.thd_positions(cu_seqlens, tokens, offset)
+
+
+def _rope_q_rows(t3, cos, sin, emb_offset, emb_dim, pairing, positions, batch, inverse):
+    pe = t3[:, :, emb_offset: emb_offset + emb_dim]
+    ops.rope_rows(pe, pe, cos, sin, pairing, pairing, inverse, positions, batch)
+
+
+def _rope_q_forward(ctx, pairing, q, cos, sin, qk_head_dim, emb_dim, cu_seqlens_q, cp_rank, cp_size, emb_offset, sp_offset):
+    if emb_offset is None:
+        emb_offset = qk_head_dim
+    if cu_seqlens_q is None:       # sbhd
+        batch, nheads, headdim = q.shape[1], q.shape[2], q.shape[3]
+        q3 = q.view(-1, nheads, headdim)
+    else:                          # thd
+        batch, headdim = 1, q.shape[2]
+        q3 = q
+    assert q3.stride(-1) == 1
+    assert cos.is_contiguous() and sin.is_contiguous()
+    assert headdim == qk_head_dim + emb_dim
+    assert emb_dim % 4 == 0
+    positions = _token_positions(cu_seqlens_q, q3.shape[0], cp_rank, cp_size, sp_offset)
+    _rope_q_rows(q3, cos, sin, emb_offset, emb_dim, pairing, positions, batch, False)
+    ctx.mark_dirty(q)
+    ctx.save_for_backward(cos, sin)
+    ctx.args = (emb_offset, emb_dim, positions, batch)
+    return q
+
+
+def _rope_q_backward(ctx, pairing, grad):
+    cos, sin = ctx.saved_tensors
+    emb_offset, emb_dim, positions, batch = ctx.args
+    grad = grad.contiguous()
+    _rope_q_rows(grad.view(-1, grad.shape[-2], grad.shape[-1]), cos, sin, emb_offset, emb_dim, pairing, positions, batch, True)
+    return grad, None, None, None, None, None, None, None, None, None
+
+
+class ApplyMLARotaryEmbQInterleaved(torch.autograd.Function):
+    """Interleaved rotary embedding of MLA's query, in place (reference: dsa_fused_kernels.py:230-349):
+    pairs are (x[2i], x[2i+1]) and stay where they are."""
+
+    @staticmethod
+    def forward(ctx, q, cos, sin, qk_head_dim, emb_dim, cu_seqlens_q, cp_rank, cp_size, emb_offset=None, sp_offset=0):
+        return _rope_q_forward(ctx, ops.ROPE_ADJACENT, q, cos, sin, qk_head_dim, emb_dim, cu_seqlens_q, cp_rank, cp_size,
+                               emb_offset, sp_offset)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return _rope_q_backward(ctx, ops.ROPE_ADJACENT, grad)
+
+
+class ApplyMLARotaryEmbQNonInterleavedWithOffset(torch.autograd.Function):
+    """Rotary embedding of MLA's query with pairs (x[i], x[i + emb_dim/2]), in place
+    (reference: dsa_fused_kernels.py:501-603)."""
+
+    @staticmethod
+    def forward(ctx, q, cos, sin, qk_head_dim, emb_dim, cu_seqlens_q, cp_rank, cp_size, emb_offset=None, sp_offset=0):
+        return _rope_q_forward(ctx, ops.ROPE_SPLIT, q, cos, sin, qk_head_dim, emb_dim, cu_seqlens_q, cp_rank, cp_size,
+                               emb_offset, sp_offset)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return _rope_q_backward(ctx, ops.ROPE_SPLIT, grad)
+
+
+def fused_apply_mla_rope(t, cos, sin, qk_head_dim: int, emb_dim: int, cu_seqlens_q=None, cp_rank: int = 0,
+                         cp_size: int = 1, rotary_interleaved: bool = False, pe_first: bool = False, sp_offset: int = 0):
+    """Rotary embedding of MLA's query, modifying ``t`` in place (reference: dsa_fused_kernels.py:1168-1212).
+
+    ``t``: [seq, batch, heads, qk_head_dim + emb_dim] or packed [tokens, heads, ...]; cos / sin
+    [max_seq_len, 1, 1, emb_dim]; ``pe_first`` puts the rotary columns at the front of a head.
+    """
+    emb_offset = 0 if pe_first else qk_head_dim
+    fn = ApplyMLARotaryEmbQInterleaved if rotary_interleaved else ApplyMLARotaryEmbQNonInterleavedWithOffset
+    return fn.apply(t, cos, sin, qk_head_dim, emb_dim, cu_seqlens_q, cp_rank, cp_size, emb_offset, sp_offset)
+
+
+class FusedRopePermuteCat(torch.autograd.Function):
+    """``query[s, b, h, :] = cat(q_content[h, s*b, :], rope(q_pos_emb[s, b, h, :]))`` in one pass
+    (reference: dsa_fused_kernels.py:1010-1131).  The rotary input pairs are adjacent elements; the
+    output keeps them adjacent (interleaved) or splits them into halves (non-interleaved)."""
+
+    @staticmethod
+    def forward(ctx, q_content, q_pos_emb, cos, sin, cu_seqlens_q, cp_rank, cp_size, rotary_interleaved=False):
+        if q_pos_emb.ndim == 4:
+            s, b, nheads, emb_dim = q_pos_emb.shape
+            S = s * b
+        else:
+            S, nheads, emb_dim = q_pos_emb.shape
+            s, b = S, 1
+        d_out = q_content.shape[-1]
+        qc = q_content.reshape(nheads, S, d_out)
+        pe = q_pos_emb.reshape(S, nheads, emb_dim)
+        out = q_content.new_empty(S, nheads, d_out + emb_dim)
+        positions = _token_positions(cu_seqlens_q, S, cp_rank, cp_size)
+        out_pairing = ops.ROPE_ADJACENT if rotary_interleaved else ops.ROPE_SPLIT
+        ops.rope_rows(pe, out[:, :, d_out:], cos, sin, ops.ROPE_ADJACENT, out_pairing, False, positions, b,
+                      main_src=qc.transpose(0, 1), main_dst=out[:, :, :d_out])
+        ctx.save_for_backward(cos, sin)
+        ctx.args = (s, b, nheads, d_out, emb_dim, positions, out_pairing, q_content.shape, q_pos_emb.ndim)
+        return out.view(s, b, nheads, d_out + emb_dim) if q_pos_emb.ndim == 4 else out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        cos, sin = ctx.saved_tensors
+        s, b, nheads, d_out, emb_dim, positions, out_pairing, qc_shape, pe_ndim = ctx.args
+        S = s * b
+        g = grad_output.reshape(S, nheads, d_out + emb_dim).contiguous()
+        grad_qc = g.new_empty(nheads, S, d_out)
+        grad_pe = g.new_empty(S, nheads, emb_dim)
+        ops.rope_rows(g[:, :, d_out:], grad_pe, cos, sin, out_pairing, ops.ROPE_ADJACENT, True, positions, b,
+                      main_src=g[:, :, :d_out], main_dst=grad_qc.transpose(0, 1))
+        grad_qc = grad_qc.view(qc_shape)
+        if pe_ndim == 4:
+            grad_pe = grad_pe.view(s, b, nheads, emb_dim)
+        return grad_qc, grad_pe, None, None, None, None, None, None
+
+
+def fused_rope_permute_cat(q_content, q_pos_emb, cos, sin, cu_seqlens_q=None, cp_rank: int = 0, cp_size: int = 1,
+                           rotary_interleaved: bool = False):
+    """Permute ``q_content`` (HSD -> SBHD), apply the rotary embedding to ``q_pos_emb`` and concatenate
+    (reference: dsa_fused_kernels.py:1134-1165)."""
+    return FusedRopePermuteCat.apply(q_content, q_pos_emb, cos, sin, cu_seqlens_q, cp_rank, cp_size, rotary_interleaved)
+
+
+class ApplyMLARotaryEmbAbsorbKV(torch.autograd.Function):
+    """``key[t, h, :] = cat(kv[t, h, :k_dim], rope(k_pos_emb[t, :]))``: the shared rotary part of the
+    key is rotated once per token and broadcast to every head (reference: dsa_fused_kernels.py:1610-1793)."""
+
+    @staticmethod
+    def forward(ctx, kv, k_pos_emb, cos, sin, emb_dim, k_dim, cu_seqlens_kv, cp_rank, cp_size, rotary_interleaved=False):
+        if cu_seqlens_kv is None:
+            max_seqlen, batch, nheads, headdim = kv.shape
+            kv3 = kv.view(-1, nheads, headdim)
+        else:
+            max_seqlen, batch = None, 1
+            kv3 = kv
+            nheads, headdim = kv.shape[1], kv.shape[2]
+        T = kv3.shape[0]
+        emb2 = k_pos_emb.reshape(T, emb_dim)
+        assert headdim == k_dim
+        assert kv3.stride(-1) == 1 and emb2.stride(-1) == 1
+        assert cos.is_contiguous() and sin.is_contiguous()
+        assert emb_dim % 4 == 0
+        o_key = kv.new_empty(T, nheads, emb_dim + k_dim)
+        positions = _token_positions(cu_seqlens_kv, T, cp_rank, cp_size)
+        out_pairing = ops.ROPE_ADJACENT if rotary_interleaved else ops.ROPE_SPLIT
+        ops.rope_rows(emb2.unsqueeze(1).expand(T, nheads, emb_dim), o_key[:, :, k_dim:], cos, sin, ops.ROPE_ADJACENT,
+                      out_pairing, False, positions, batch, main_src=kv3, main_dst=o_key[:, :, :k_dim])
+        ctx.save_for_backward(cos, sin)
+        ctx.args = (emb_dim, k_dim, positions, batch, out_pairing, max_seqlen)
+        if cu_seqlens_kv is None:
+            o_key = o_key.view(max_seqlen, -1, nheads, emb_dim + k_dim)
+        return o_key
+
+    @staticmethod
+    def backward(ctx, dk):
+        cos, sin = ctx.saved_tensors
+        emb_dim, k_dim, positions, batch, out_pairing, max_seqlen = ctx.args
+        nheads = dk.shape[-2]
+        dk3 = dk.contiguous().view(-1, nheads, emb_dim + k_dim)
+        T = dk3.shape[0]
+        d_kv = dk3.new_empty(T, nheads, k_dim)
+        ops.rope_rows(None, None, None, None, 0, 0, main_src=dk3[:, :, :k_dim], main_dst=d_kv)
+        d_emb = ops.rope_headsum_inverse(dk3[:, :, k_dim:], cos, sin, out_pairing, positions, batch).view(T, 1, emb_dim)
+        if max_seqlen is not None:
+            d_kv = d_kv.view(max_seqlen, batch, nheads, k_dim)
+            d_emb = d_emb.view(max_seqlen, batch, 1, emb_dim)
+        return d_kv, d_emb, None, None, None, None, None, None, None, None
+
+
+def fused_apply_mla_rope_for_absorb_kv(kv, k_pos_emb, cos, sin, emb_dim: int, k_dim: int, cu_seqlens_kv=None,
+                                       cp_rank: int = 0, cp_size: int = 1, rotary_interleaved: bool = False):
+    """Key rows of the absorbed MLA form: copy of ``kv`` plus the rotated, head-shared ``k_pos_emb``
+    (reference: dsa_fused_kernels.py:1796-1841)."""
+    return ApplyMLARotaryEmbAbsorbKV.apply(kv, k_pos_emb, cos, sin, emb_dim, k_dim, cu_seqlens_kv, cp_rank, cp_size,
+                                           rotary_interleaved)

@@ -391,3 +391,100 @@ def _(p_out, sm_scale):
 def attn_dist(p_out, sm_scale: float):
     """fp32 ``[S,K]``: mean over heads of softmax over slots of ``p_out * sm_scale``."""
     return _attn_dist_op(p_out, float(sm_scale))
+
+
+# --------------------------------------------------------------------------------------------
+# rotary position embedding fused with the surrounding copies
+# --------------------------------------------------------------------------------------------
+ROPE_ADJACENT, ROPE_SPLIT = 0, 1   # where pair i sits in a row: (2i, 2i+1) or (i, i + emb_dim/2)
+
+
+def _rows_view(t: torch.Tensor, what: str):
+    """(data_ptr, token stride, head stride) of a [tokens, heads, width] bf16 view with unit inner stride."""
+    if t.dtype != torch.bfloat16 or t.ndim != 3 or (t.shape[-1] > 1 and t.stride(-1) != 1):
+        raise ValueError("%s must be a bf16 [tokens, heads, width] view with unit inner stride" % what)
+    return t.data_ptr(), t.stride(0), t.stride(1)
+
+
+def _cos_sin(cos: torch.Tensor, sin: torch.Tensor, emb_dim: int):
+    cos2, sin2 = cos.reshape(-1, emb_dim), sin.reshape(-1, emb_dim)
+    if cos2.dtype not in (torch.float32, torch.bfloat16):
+        cos2, sin2 = cos2.float(), sin2.float()
+    if sin2.dtype != cos2.dtype:
+        sin2 = sin2.to(cos2.dtype)
+    return _c(cos2), _c(sin2)
+
+
+def thd_positions(cu_seqlens: torch.Tensor, tokens: int, offset: int = 0) -> torch.Tensor:
+    """Position of every packed token inside its own sequence (int32 [tokens]); token t of the call
+    is global token t + offset.  Tokens past the last sequence get position 0."""
+    cu = cu_seqlens.to(torch.int64)
+    t = torch.arange(tokens, device=cu.device, dtype=torch.int64) + int(offset)
+    seq = torch.searchsorted(cu[1:].contiguous(), t, right=True)
+    inside = seq < cu.numel() - 1
+    start = cu[seq.clamp(max=cu.numel() - 2)]
+    return torch.where(inside, t - start, torch.zeros_like(t)).to(torch.int32)
+
+
+def rope_rows(pe_src: Optional[torch.Tensor], pe_dst: Optional[torch.Tensor], cos: Optional[torch.Tensor],
+              sin: Optional[torch.Tensor], in_pairing: int, out_pairing: int, inverse: bool = False,
+              positions: Optional[torch.Tensor] = None, batch: int = 1,
+              main_src: Optional[torch.Tensor] = None, main_dst: Optional[torch.Tensor] = None) -> None:
+    """Rotates the pe part of every (token, head) row and copies the main part (either may be absent).
+
+    All tensors are [tokens, heads, width] bf16 views (any token / head strides, rows starting on
+    16-byte boundaries); ``pe_src`` may be ``pe_dst`` when both pairings are equal; a head stride of 0
+    in ``pe_src`` broadcasts one row.  cos / sin: [positions, emb_dim] fp32 or bf16.  Writes in place
+    into ``pe_dst`` / ``main_dst``.
+    """
+    ref = pe_dst if pe_dst is not None else main_dst
+    _need_gpu(pe_src, pe_dst, cos, sin, positions, main_src, main_dst)
+    tokens, heads = ref.shape[0], ref.shape[1]
+    emb = 0
+    ps = pd = (None, 0, 0)
+    cos2 = sin2 = None
+    if pe_dst is not None:
+        emb = pe_dst.shape[-1]
+        if pe_src.shape != pe_dst.shape:
+            raise ValueError("pe_src and pe_dst differ in shape: %s vs %s" % (tuple(pe_src.shape), tuple(pe_dst.shape)))
+        ps, pd = _rows_view(pe_src, "pe_src"), _rows_view(pe_dst, "pe_dst")
+        cos2, sin2 = _cos_sin(cos, sin, emb)
+        if positions is not None:
+            positions = _c(positions.int())
+            if positions.numel() != tokens:
+                raise ValueError("positions must hold one entry per token")
+    ms = md = (None, 0, 0)
+    d_main = 0
+    if main_dst is not None:
+        if main_src.shape != main_dst.shape or main_dst.shape[:2] != ref.shape[:2]:
+            raise ValueError("main_src / main_dst shapes do not match the pe rows")
+        d_main = main_dst.shape[-1]
+        ms, md = _rows_view(main_src, "main_src"), _rows_view(main_dst, "main_dst")
+    lib = _lib.load()
+    with torch.cuda.device(ref.device):
+        _lib.check(lib.dsa_rope_rows(ms[0], ms[1], ms[2], md[0], md[1], md[2], d_main, ps[0], ps[1], ps[2], pd[0], pd[1], pd[2],
+                                     emb, cos2.data_ptr() if emb else None, sin2.data_ptr() if emb else None,
+                                     int(emb and cos2.dtype == torch.float32),
+                                     positions.data_ptr() if (emb and positions is not None) else None, int(batch),
+                                     tokens, heads, int(in_pairing), int(out_pairing), int(bool(inverse)), _stream(ref)),
+                   "dsa_rope_rows")
+
+
+def rope_headsum_inverse(grad_pe: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, in_pairing: int,
+                         positions: Optional[torch.Tensor] = None, batch: int = 1) -> torch.Tensor:
+    """d_emb [tokens, emb_dim] bf16 = inverse rotation of bf16(sum over heads of grad_pe [tokens, heads, emb_dim])."""
+    _need_gpu(grad_pe, cos, sin, positions)
+    g = _rows_view(grad_pe, "grad_pe")
+    tokens, heads, emb = grad_pe.shape
+    cos2, sin2 = _cos_sin(cos, sin, emb)
+    if positions is not None:
+        positions = _c(positions.int())
+    d_emb = torch.empty(tokens, emb, dtype=torch.bfloat16, device=grad_pe.device)
+    lib = _lib.load()
+    with torch.cuda.device(grad_pe.device):
+        _lib.check(lib.dsa_rope_headsum_inverse(g[0], g[1], g[2], d_emb.data_ptr(), emb, emb, cos2.data_ptr(), sin2.data_ptr(),
+                                                int(cos2.dtype == torch.float32),
+                                                positions.data_ptr() if positions is not None else None, int(batch),
+                                                tokens, heads, int(in_pairing), _stream(grad_pe)),
+                   "dsa_rope_headsum_inverse")
+    return d_emb
