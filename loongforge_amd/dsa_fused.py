@@ -152,8 +152,18 @@ class DSAIndexerFused(MegatronModule):
             raise NotImplementedError("chunkpipe is not supported by the single-GPU DSA modules")
         self.indexer_kernel = DSAIndexerKernel()
 
-    def _apply_rope(self, x, rotary_pos_emb, mscale, cu_seqlens):
-        """RoPE on the leading ``qk_pos_emb_head_dim`` channels ("PE first", dsa_fused.py:453-487)."""
+    def _apply_rope(self, x, rotary_pos_emb, mscale, cu_seqlens, rotary_pos_cos=None, rotary_pos_sin=None):
+        """RoPE on the leading ``qk_pos_emb_head_dim`` channels ("PE first", dsa_fused.py:423-487): the fused
+        in-place kernel when ``config.apply_rope_fusion`` is set (:435-451), torch ops otherwise."""
+        if getattr(self.config, "apply_rope_fusion", False) and x.is_cuda:
+            from .dsa_fused_kernels import fused_apply_mla_rope
+
+            x4 = x if (cu_seqlens is not None or x.ndim == 4) else x.unsqueeze(1)
+            out = fused_apply_mla_rope(x4.contiguous(), rotary_pos_cos, rotary_pos_sin,
+                                       self.index_head_dim - self.qk_pos_emb_head_dim, self.qk_pos_emb_head_dim,
+                                       cu_seqlens, self.pg_collection.cp.rank(), self.pg_collection.cp.size(),
+                                       pe_first=True, sp_offset=0)
+            return out.view(x.shape)
         x_pe, x_nope = torch.split(
             x, [self.qk_pos_emb_head_dim, self.index_head_dim - self.qk_pos_emb_head_dim], dim=-1
         )
@@ -173,6 +183,9 @@ class DSAIndexerFused(MegatronModule):
         packed_seq = packed_seq_params is not None and packed_seq_params.qkv_format == "thd"
         rotary_pos_emb = self.rotary_pos_emb(rotary_seq_len, offset=0, packed_seq=packed_seq)
         mscale = 1.0
+        cos = sin = None
+        if getattr(self.config, "apply_rope_fusion", False):
+            cos, sin = self.rotary_pos_emb.get_cached_cos_sin(rotary_seq_len, dtype=x.dtype, packed_seq=packed_seq)
         if packed_seq_params is not None:
             cu_seqlens_q = packed_seq_params.cu_seqlens_q_padded
             if cu_seqlens_q is None:
@@ -185,16 +198,16 @@ class DSAIndexerFused(MegatronModule):
 
         q, _ = self.linear_wq_b(qr)
         q = q.view(*q.size()[:-1], self.index_n_heads, self.index_head_dim)
-        q = self._apply_rope(q, rotary_pos_emb, mscale, cu_seqlens_q)
+        q = self._apply_rope(q, rotary_pos_emb, mscale, cu_seqlens_q, cos, sin)
 
         k, _ = self.linear_wk(x)
         k = self.k_norm(k)
         if packed_seq_params is None:
             k = k.unsqueeze(-2)
-            k = self._apply_rope(k, rotary_pos_emb, mscale, cu_seqlens_kv)
+            k = self._apply_rope(k, rotary_pos_emb, mscale, cu_seqlens_kv, cos, sin)
             k = k.squeeze(-2)
         else:
-            k = self._apply_rope(k.unsqueeze(-2), rotary_pos_emb, mscale, cu_seqlens_kv).squeeze(-2)
+            k = self._apply_rope(k.unsqueeze(-2), rotary_pos_emb, mscale, cu_seqlens_kv, cos, sin).squeeze(-2)
 
         if getattr(self.config, "dsa_indexer_rotate_activation", True) and not defer_rotation:
             q = rotate_activation(q)

@@ -107,6 +107,12 @@ class RotaryEmbedding(torch.nn.Module):
         return emb[:, None, None, :]
 
 
+    def get_cached_cos_sin(self, max_seq_len, dtype=torch.float32, packed_seq=False):
+        """``(cos, sin)`` of the angles, each ``[seq, 1, 1, dim]`` in ``dtype`` (what the fused rotary kernels take)."""
+        emb = self.forward(max_seq_len, packed_seq=packed_seq)
+        return emb.cos().to(dtype).contiguous(), emb.sin().to(dtype).contiguous()
+
+
 def _rotate_half(x, interleaved):
     if not interleaved:
         x1, x2 = torch.chunk(x, 2, dim=-1)

@@ -153,3 +153,50 @@ def test_fused_attention_module_matches_oracle_pipeline(gpu):
     grads = {n: p.grad for n, p in mod.named_parameters()}
     assert all(gv is not None and torch.isfinite(gv).all() and gv.abs().max() > 0 for n, gv in grads.items()
                if "indexer" in n and "k_norm.bias" not in n)
+
+
+def test_indexer_front_end_with_fused_rope_matches_the_torch_rope(gpu):
+    """config.apply_rope_fusion routes the indexer's RoPE through the in-place HIP kernel
+    (dsa_fused.py:435-451 of the reference); q and k must agree with the torch-op path to bf16 rounding,
+    for one sequence and for a packed batch, and gradients must reach the projection weights."""
+    import copy
+
+    from loongforge_amd import dsa_fused
+    from loongforge_amd.megatron_compat import PackedSeqParams
+
+    S, Hi, Di, hid, qlr = 300, 4, 128, 96, 48
+    cfg = _cfg(num_attention_heads=16, hidden_size=hid, q_lora_rank=qlr, dsa_indexer_n_heads=Hi, dsa_indexer_head_dim=Di,
+               dsa_indexer_topk=64, dsa_indexer_loss_coeff=1.0, rope_type="rope", rotary_percent=1.0, rotary_base=10000,
+               init_method=None, layernorm_epsilon=1e-5, dsa_indexer_rotate_activation=True, enable_chunkpipe=False)
+    sub = dsa_fused.DSAIndexerFusedSubmodules(linear_wq_b=_Linear, linear_wk=_Linear, k_norm=_Norm, linear_weights_proj=_Linear)
+    torch.manual_seed(1)
+    plain = dsa_fused.DSAIndexerFused(cfg, sub)
+    for p in plain.parameters():
+        if p.ndim == 2:
+            torch.nn.init.normal_(p, std=p.shape[1] ** -0.5)
+    plain = plain.to(gpu)
+    fused = copy.deepcopy(plain)
+    fused.config = copy.copy(cfg)
+    fused.config.apply_rope_fusion = True
+    g = torch.Generator().manual_seed(2)
+    for packed in (False, True):
+        shape = (S, hid) if packed else (S, 1, hid)
+        x = torch.randn(*shape, generator=g).to(torch.bfloat16).to(gpu)
+        qr = torch.randn(*shape[:-1], qlr, generator=g).to(torch.bfloat16).to(gpu)
+        psp = None
+        if packed:
+            cu = torch.tensor([0, 100, 101, 300], dtype=torch.int32, device=gpu)
+            psp = PackedSeqParams(qkv_format="thd", cu_seqlens_q=cu, cu_seqlens_kv=cu, max_seqlen_q=199, max_seqlen_kv=199)
+        q0, k0, w0 = plain.get_query_key_weight_tensors(x, qr, psp, defer_rotation=True)
+        q1, k1, w1 = fused.get_query_key_weight_tensors(x, qr, psp, defer_rotation=True)
+        assert q1.shape == q0.shape and k1.shape == k0.shape and torch.equal(w0, w1)
+        for a, b in ((q1, q0), (k1, k0)):
+            err = (a.float() - b.float()).abs()
+            # the torch path rounds every product and the sum to bf16, the kernel once: a few units in the last
+            # place of the larger of the result and its two terms (inputs here stay below 8 in magnitude)
+            assert (err <= 2.0 ** -6 * (b.float().abs() + 2.0)).all()
+            assert torch.equal(a[..., 64:], b[..., 64:])                      # the non-rotary half is untouched
+        (q1.float().square().sum() + k1.float().square().sum()).backward()
+        assert all(p.grad is not None and torch.isfinite(p.grad).all() and p.grad.abs().max() > 0
+                   for n, p in fused.named_parameters() if "weights_proj" not in n and "k_norm.bias" not in n)
+        fused.zero_grad()
