@@ -28,6 +28,17 @@ def test_forward_against_oracle(gpu, S, H, K, q_start, skv, seed):
     assert (lse.cpu() - rl).abs().max().item() < 1e-4
 
 
+@pytest.mark.parametrize("K", [4096, 8192])
+def test_forward_with_a_top_k_beyond_2048(gpu, K):
+    """Wider slot lists run with a three-stage tile ring; the backward is limited to 2048 slots."""
+    skv = K + 1500
+    inp = O.make_mla_inputs(48, 64, K, seed=11, skv=skv, q_start=skv - 48)
+    out, lse, _ = _run_fwd(inp, gpu, skv - 48)
+    ro, rl, _ = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, skv - 48, inp.sm_scale, 512)
+    assert_close(out, ro, "out")
+    assert (lse.cpu() - rl).abs().max().item() < 1e-4
+
+
 def test_forward_p_out_and_attn_dist(gpu):
     from loongforge_amd import ops
     from loongforge_amd.dsa_fused_kernels import triton_attn_dist
