@@ -171,6 +171,22 @@ def main():
     e2.record()
     torch.cuda.synchronize()
     t_logits, t_topk = e0.elapsed_time(e1), e1.elapsed_time(e2)
+    # the remaining kernels of the path, once each after an untimed call: indexer backward on the
+    # selected logits, and the head-averaged attention distribution over the forward's raw logits
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        a, b = ev(), ev()
+        a.record()
+        r = fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b), r
+    g_sel = torch.empty(S, K, dtype=torch.float32, device=dev).normal_()
+    t_ibwd, _ = timed(lambda: ops.indexer_bwd(g_sel, q8, k8, ksc, wsd, ids))
+    _, _, p_raw = ops.sparse_mla_fwd(q, kv, idx, 0, inp.sm_scale, DV, True)
+    t_dist, _ = timed(lambda: ops.attn_dist(p_raw, inp.sm_scale))
+    del p_raw, g_sel
     # one forward with cold caches (a 1 GiB fill evicts L2 and the memory-side cache first)
     flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     flush.fill_(1)
@@ -266,6 +282,9 @@ def main():
         "indexer_topk_frac_of_fp8_peak": round(flops_idx / (t_idx * 1e-3) / 1e12 / PEAK_FP8, 4),
         "indexer_logits_ms": round(t_logits, 3), "topk_ms": round(t_topk, 3),
         "topk_hbm_gbps": round((4.0 * vis + 8.0 * S * K) / (t_topk * 1e-3) / 1e9, 1),
+        "indexer_bwd_ms": round(t_ibwd, 3),
+        "attn_dist_ms": round(t_dist, 3),
+        "attn_dist_gbps": round((2.0 * S * H * K + 4.0 * S * K) / (t_dist * 1e-3) / 1e9, 1),
         "mla_fwd_ms_cold_caches": round(t_fwd_cold, 3),
         "mla_fwd_gather_gbps": round(2.0 * DQK * pairs / (t_fwd * 1e-3) / 1e9, 1),
         "nominal": {"note": "the same times priced on S*K pairs and S*S logits, as the reference's own print-outs do",

@@ -1,6 +1,8 @@
 // Head-averaged softmax over the selected slots: target[i,t] = mean_h softmax_t(p_out[i,h,:] * c).
 // HBM-bound: reads H*K logits per query once.  One workgroup per query; each wave takes heads
-// w, w+4, ...; a head's K logits live in registers (K/64 per lane), so p_out is read exactly once.
+// w, w+4, ...; a head's K logits live in registers, so p_out is read exactly once.  Two variants:
+// 16-byte loads when the layout allows it, element loads otherwise (the same arithmetic; the partial
+// sums of a head are grouped differently, so results agree to fp32 rounding, not bit for bit).
 #include "dsa_common.h"
 
 namespace {
@@ -62,11 +64,108 @@ __global__ __launch_bounds__(256) void attn_dist_kernel(const void* __restrict__
     target[i * K + t] = ((acc_s[t] + acc_s[K + t]) + (acc_s[2 * K + t] + acc_s[3 * K + t])) * invh;
 }
 
+// The same with 16-byte loads: lane l of a wave owns slots 8 (64 v + l) .. +7 of every head.  Needs
+// K, the strides and the base address to be multiples of 8 elements.
+template <bool F32, int NC>
+__global__ __launch_bounds__(256) void attn_dist_vec_kernel(const void* __restrict__ p_out, int H, int K,
+                                                            int64_t ld_s, int64_t ld_h, float c2,
+                                                            float* __restrict__ target) {
+  extern __shared__ float acc_s[];            // [4 waves][K]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t i = blockIdx.x;
+  float acc[NC][8];
+#pragma unroll
+  for (int v = 0; v < NC; v++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[v][e] = 0.f;
+  // raw 16-byte pieces of one head; the next head's are requested before this head's arithmetic
+  struct Raw { uint4 a[NC]; uint4 b[NC]; };
+  auto fetch = [&](int h, Raw& r) {
+    const int64_t base = i * ld_s + h * ld_h;
+#pragma unroll
+    for (int v = 0; v < NC; v++) {
+      const int t = 8 * (v * 64 + lane);
+      if (t < K && h < H) {
+        if (F32) {
+          r.a[v] = *(const uint4*)((const float*)p_out + base + t);
+          r.b[v] = *(const uint4*)((const float*)p_out + base + t + 4);
+        } else {
+          r.a[v] = *(const uint4*)((const unsigned short*)p_out + base + t);
+        }
+      }
+    }
+  };
+  Raw cur, nxt;
+  fetch(wave, cur);
+  for (int h = wave; h < H; h += 4) {
+    fetch(h + 4, nxt);
+    float z[NC][8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < NC; v++) {
+      const int t = 8 * (v * 64 + lane);
+      if (t < K) {
+        if (F32) {
+          const unsigned w[8] = {cur.a[v].x, cur.a[v].y, cur.a[v].z, cur.a[v].w, cur.b[v].x, cur.b[v].y, cur.b[v].z, cur.b[v].w};
+#pragma unroll
+          for (int e = 0; e < 8; e++) z[v][e] = __builtin_bit_cast(float, w[e]) * c2;
+        } else {
+          const unsigned w[4] = {cur.a[v].x, cur.a[v].y, cur.a[v].z, cur.a[v].w};
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            z[v][2 * e] = __builtin_bit_cast(float, w[e] << 16) * c2;
+            z[v][2 * e + 1] = __builtin_bit_cast(float, w[e] & 0xffff0000u) * c2;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) z[v][e] = -INFINITY;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e++) mx = fmaxf(mx, z[v][e]);
+    }
+    cur = nxt;
+    mx = wave_max(mx);
+    if (mx == -INFINITY) continue;            // head with no valid slot contributes nothing
+    float sum = 0.f;
+#pragma unroll
+    for (int v = 0; v < NC; v++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) { z[v][e] = exp2f(z[v][e] - mx); sum += z[v][e]; }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int v = 0; v < NC; v++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc[v][e] += z[v][e] * inv;
+  }
+#pragma unroll
+  for (int v = 0; v < NC; v++) {
+    const int t = 8 * (v * 64 + lane);
+    if (t < K) {
+      *(f32x4*)(acc_s + wave * K + t) = f32x4{acc[v][0], acc[v][1], acc[v][2], acc[v][3]};
+      *(f32x4*)(acc_s + wave * K + t + 4) = f32x4{acc[v][4], acc[v][5], acc[v][6], acc[v][7]};
+    }
+  }
+  __syncthreads();
+  const float invh = 1.0f / (float)H;
+  for (int t = threadIdx.x; t < K; t += 256)
+    target[i * K + t] = ((acc_s[t] + acc_s[K + t]) + (acc_s[2 * K + t] + acc_s[3 * K + t])) * invh;
+}
+
 template <bool F32>
 int launch(const void* p_out, int S, int H, int K, int64_t ld_s, int64_t ld_h, float sm_scale, float* target,
            hipStream_t st) {
   const float c2 = sm_scale * 1.4426950408889634f;
   size_t smem = (size_t)4 * K * sizeof(float);
+  const bool vec = K % 8 == 0 && ld_s % 8 == 0 && ld_h % 8 == 0 && ((uintptr_t)p_out % 32) == 0;
+  if (vec) {
+    const int nc = (K + 511) / 512;
+#define DSA_ADV_CASE(N) \
+    if (nc <= N) { attn_dist_vec_kernel<F32, N><<<dim3(S), dim3(256), smem, st>>>(p_out, H, K, ld_s, ld_h, c2, target); return 0; }
+    DSA_ADV_CASE(1) DSA_ADV_CASE(2) DSA_ADV_CASE(4) DSA_ADV_CASE(8)
+#undef DSA_ADV_CASE
+  }
   int nv = (K + 63) / 64;
 #define DSA_AD_CASE(N) \
   if (nv <= N) { attn_dist_kernel<F32, N><<<dim3(S), dim3(256), smem, st>>>(p_out, H, K, ld_s, ld_h, c2, target); return 0; }
