@@ -23,7 +23,13 @@ constexpr int D = 128;
 constexpr int TK = 128;                 // slots per tile
 constexpr int TILE_BYTES = TK * D;      // fp8 key rows
 constexpr int RED_STRIDE = 132;         // floats per head row of the cross-wave reduction buffer
-constexpr int STRIP_STRIDE = 144;       // bytes per key row of the d_k transpose strip (128 + bank spread)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned cvt_pk_bf16(float lo, float hi) {    // one v_cvt_pk_bf16_f32
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
+constexpr int STRIP_STRIDE = 136;       // bytes per key row of the d_k transpose strip (two d-tiles of 64 bytes + bank spread)
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
 
@@ -56,7 +62,7 @@ template <int NHT>
 __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
     const float* __restrict__ gsc, const unsigned char* __restrict__ q8, const unsigned char* __restrict__ k8,
     const float* __restrict__ k_scale, const float* __restrict__ q_w, const int* __restrict__ ids,
-    const int* __restrict__ dst, float* __restrict__ rows, float* __restrict__ d_q8, float* __restrict__ d_qw,
+    const int* __restrict__ dst, unsigned short* __restrict__ rows, float* __restrict__ d_q8, float* __restrict__ d_qw,
     int q0, int cnt, int Sk, int K, int dummy_row) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int HI = 32 * NHT;
@@ -227,40 +233,41 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
 
     // ---- d_k8 rows: row^T[d, key] = Q^T . E, 32 keys of this wave --------------------------------
     {
-      // The 32 x 32 fp32 block of a d-tile is transposed through a wave-private LDS strip, so that a
-      // store instruction writes eight complete 128-byte row segments (lane: key 8*i + lane/8,
-      // 16-byte piece lane%8) instead of 32 scattered 32-byte pieces.
-      float* rowp[4];
+      // Rows leave as bf16 (the ordered sum over a key's rows runs in fp32; one row carries 2^-9 of
+      // relative rounding, so E enters these products as its bf16 head alone).  Two 32 x 32 d-tiles at a
+      // time are rounded, transposed through a wave-private LDS strip and stored, so that a store
+      // instruction writes eight complete 128-byte row segments (lane: key 8*i + lane/8, 16-byte piece
+      // lane%8) instead of scattered 8-byte pieces.
+      unsigned short* rowp[4];
 #pragma unroll
       for (int i = 0; i < 4; i++)
-        rowp[i] = rows + (size_t)dst_s[t * TK + 32 * wave + 8 * i + (lane >> 3)] * D + 4 * (lane & 7);
-      unsigned char* sw = strip + r * STRIP_STRIDE + 16 * g;
+        rowp[i] = rows + (size_t)dst_s[t * TK + 32 * wave + 8 * i + (lane >> 3)] * D + 8 * (lane & 7);
+      unsigned char* sw = strip + r * STRIP_STRIDE + 8 * g;
       const unsigned char* sr = strip + (lane >> 3) * STRIP_STRIDE + (lane & 7) * 16;
       auto row_mfmas = [&](int dt, f32x16& racc) {
         mfma_v_av_first(racc, qt[dt][0], ehi[0][0]);
-        mfma_v_av(racc, qt[dt][0], elo[0][0]);
 #pragma unroll
-        for (int kk = 1; kk < 2 * NHT; kk++) {
-          mfma_v_av(racc, qt[dt][kk], ehi[kk >> 1][kk & 1]);
-          mfma_v_av(racc, qt[dt][kk], elo[kk >> 1][kk & 1]);
-        }
+        for (int kk = 1; kk < 2 * NHT; kk++) mfma_v_av(racc, qt[dt][kk], ehi[kk >> 1][kk & 1]);
       };
       f32x16 racc[2];
       row_mfmas(0, racc[0]);
 #pragma unroll
       for (int dt = 0; dt < 4; dt++) {
-        // the next d-tile's MFMAs run while this one goes through the strip and out to memory
+        // the next d-tile's MFMAs run while this one is rounded into the strip
         if (dt + 1 < 4) row_mfmas(dt + 1, racc[(dt + 1) & 1]);
         else mfma_done_v(racc[dt & 1]);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          const f32x4 w = {racc[dt & 1][4 * j], racc[dt & 1][4 * j + 1], racc[dt & 1][4 * j + 2], racc[dt & 1][4 * j + 3]};
-          *(f32x4*)(sw + 32 * j) = w;                // d = 32*dt + 8*j + 4*g .. +3 of key r
+        for (int j = 0; j < 4; j++) {                // d = 32*dt + 8*j + 4*g .. +3 of key r
+          const uint2 w = make_uint2(cvt_pk_bf16(racc[dt & 1][4 * j], racc[dt & 1][4 * j + 1]),
+                                     cvt_pk_bf16(racc[dt & 1][4 * j + 2], racc[dt & 1][4 * j + 3]));
+          *(uint2*)(sw + 64 * (dt & 1) + 16 * j) = w;
         }
-        __builtin_amdgcn_wave_barrier();
+        if (dt & 1) {
+          __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int i = 0; i < 4; i++) *(f32x4*)(rowp[i] + 32 * dt) = *(const f32x4*)(sr + 8 * i * STRIP_STRIDE);
-        __builtin_amdgcn_wave_barrier();
+          for (int i = 0; i < 4; i++) *(uint4*)(rowp[i] + 64 * (dt >> 1)) = *(const uint4*)(sr + 8 * i * STRIP_STRIDE);
+          __builtin_amdgcn_wave_barrier();
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -365,19 +372,32 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
   if (tid < HI) d_qw[(size_t)qi * HI + tid] = (dw_red[tid] + dw_red[64 + tid]) + (dw_red[128 + tid] + dw_red[192 + tid]);
 }
 
-// d_k8[key] (+)= sum of the key's rows, ascending query order; 128 threads = 32 float4 columns x 4 row groups
-__global__ __launch_bounds__(128) void indexer_reduce_kernel(const float* __restrict__ rows, const int* __restrict__ start,
+// d_k8[key] (+)= sum of the key's bf16 rows in fp32, ascending query order; 128 threads = 16 chunks of 8
+// columns x 8 row groups (row r of the segment goes to group r % 8), the groups combined in a fixed order
+__global__ __launch_bounds__(128) void indexer_reduce_kernel(const unsigned short* __restrict__ rows, const int* __restrict__ start,
                                                              float* __restrict__ d_k8, int accumulate) {
-  __shared__ f32x4 part[4][32];
-  const int key = blockIdx.x, ch = threadIdx.x & 31, grp = threadIdx.x >> 5;
+  __shared__ float part[8][D];
+  const int key = blockIdx.x, ch = threadIdx.x & 15, grp = threadIdx.x >> 4;
   const int s0 = start[key], s1 = start[key + 1];
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int rr = s0 + grp; rr < s1; rr += 4) acc += *(const f32x4*)(rows + (size_t)rr * D + 4 * ch);
-  part[grp][ch] = acc;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) acc[e] = 0.f;
+  for (int rr = s0 + grp; rr < s1; rr += 8) {
+    const uint4 v = *(const uint4*)(rows + (size_t)rr * D + 8 * ch);
+    const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      acc[2 * e] += __builtin_bit_cast(float, w[e] << 16);
+      acc[2 * e + 1] += __builtin_bit_cast(float, w[e] & 0xffff0000u);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++) part[grp][8 * ch + e] = acc[e];
   __syncthreads();
-  if (grp == 0) {
-    f32x4 s = (part[0][ch] + part[1][ch]) + (part[2][ch] + part[3][ch]);
-    f32x4* p = (f32x4*)(d_k8 + (size_t)key * D + 4 * ch);
+  {
+    const int c = threadIdx.x;      // one column per thread
+    float s = ((part[0][c] + part[1][c]) + (part[2][c] + part[3][c])) + ((part[4][c] + part[5][c]) + (part[6][c] + part[7][c]));
+    float* p = d_k8 + (size_t)key * D + c;
     if (accumulate) s += *p;
     *p = s;
   }
@@ -398,7 +418,7 @@ Plan layout_plan(int chunk, int Sk, int K) {
   p.off_count = o; o = align_up(o + (size_t)(Sk + 1) * 4);
   p.off_start = o; o = align_up(o + (size_t)(Sk + 1) * 4);
   p.off_dst = o; o = align_up(o + (size_t)chunk * K * 4);
-  p.off_rows = o; o = align_up(o + ((size_t)chunk * K + 1) * D * 4);
+  p.off_rows = o; o = align_up(o + ((size_t)chunk * K + 1) * D * 2);
   p.total = o;
   return p;
 }
@@ -442,7 +462,7 @@ extern "C" int dsa_indexer_bwd(const float* g, const void* q8, const void* k8, c
   int* count = (int*)(ws + p.off_count);
   int* start = (int*)(ws + p.off_start);
   int* dstp = (int*)(ws + p.off_dst);
-  float* rows = (float*)(ws + p.off_rows);
+  unsigned short* rows = (unsigned short*)(ws + p.off_rows);
   size_t smem = (size_t)2 * TILE_BYTES + 4 * 32 * 256 + 4 * 2 * 32 * 128 + (size_t)K * 12 + 4 * 64 * 4 + 4 * 32 * STRIP_STRIDE;
   const size_t red_bytes = (size_t)Hi * RED_STRIDE * 4;
   if (red_bytes > (size_t)2 * TILE_BYTES + 4 * 32 * 256) smem += red_bytes;

@@ -165,7 +165,7 @@ def test_packed_32k_pipeline(gpu):
     ek = (d_k8.double().cpu() - rk).abs().masked_fill(amb_key[:, None], 0)
     ew = (d_qw[seld].double().cpu() - rw).abs()
     assert eq.max().item() <= 1e-4 * rq.abs().max().item()
-    assert ek.max().item() <= 1e-4 * rk.abs().max().item()
+    assert ek.max().item() <= 4e-3 * rk.abs().max().item()       # a key's rows are summed in fp32 from bf16 rows
     assert ew.max().item() <= 1e-4 * rw.abs().max().item()
     rest = torch.ones(T, dtype=torch.bool, device=gpu)
     rest[seld] = False

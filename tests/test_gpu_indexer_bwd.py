@@ -45,7 +45,7 @@ def test_indexer_bwd_against_oracle(gpu, S, Hi, K, seed):
     ek = (dk.double().cpu() - rk).abs().masked_fill(amb_key[:, None], 0)
     ew = (dw.double().cpu() - rw).abs()
     assert eq.max().item() <= 1e-4 * rq.abs().max().item()
-    assert ek.max().item() <= 1e-4 * rk.abs().max().item()
+    assert ek.max().item() <= 4e-3 * rk.abs().max().item()       # a key's rows are summed in fp32 from bf16 rows
     assert ew.max().item() <= 1e-4 * rw.abs().max().item()
 
 
