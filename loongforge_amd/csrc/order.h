@@ -106,16 +106,17 @@ static __global__ __launch_bounds__(1024) void key_scan_kernel(const int* __rest
 static __global__ void rank_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv, int q_start,
                             const unsigned* __restrict__ bitmap, const unsigned* __restrict__ prefix,
                             const int* __restrict__ start, int W, int* __restrict__ dst) {
-  const size_t n = (size_t)cnt * K;
-  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
-    const int ql = (int)(e / K);
-    const int v = ids[(size_t)(q0 + ql) * K + (e % K)];
+  // blockIdx.y walks the queries, blockIdx.x the slots of one query in steps of the block size
+  for (int ql = blockIdx.y; ql < cnt; ql += gridDim.y) {
+    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+    if (slot >= K) continue;
+    const int v = ids[(size_t)(q0 + ql) * K + slot];
     int d = -1;
     if (v >= 0 && v < Skv && v <= q_start + q0 + ql) {
       const size_t wi = (size_t)v * W + (ql >> 5);
       d = start[v] + (int)prefix[wi] + __popc(bitmap[wi] & ((1u << (ql & 31)) - 1u));
     }
-    dst[e] = d;
+    dst[(size_t)ql * K + slot] = d;
   }
 }
 
@@ -139,7 +140,8 @@ inline void build(const int* ids, int q0, int cnt, int K, int Skv, int q_start, 
   bm_transpose_kernel<<<dim3((W + 7) / 8, Wk), dim3(256), 0, st>>>(qmap, cnt, Skv, Wk, bitmap, W);
   bm_prefix_kernel<<<dim3((Skv + 3) / 4), dim3(256), 0, st>>>(bitmap, prefix, count, Skv, W);
   key_scan_kernel<<<dim3(1), dim3(1024), 0, st>>>(count, start, Skv);
-  rank_kernel<<<dim3(2048), dim3(256), 0, st>>>(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, start, W, dst);
+  rank_kernel<<<dim3((K + 255) / 256, cnt < 32768 ? cnt : 32768), dim3(256), 0, st>>>(ids, q0, cnt, K, Skv, q_start, bitmap, prefix,
+                                                                                     start, W, dst);
 }
 
 }  // namespace order
