@@ -3,15 +3,17 @@
 //
 //   logits[i, j] = k_scale[j] * sum_h q_w[i,h] * relu(q8[i,h,:] . k8[j,:])      ks[i] <= j < ke[i]
 //
-// One 256-thread workgroup (4 waves) owns 8 consecutive queries, two per wave, and streams the
-// keys its queries can see through LDS in tiles of 128 rows (global_load_lds, double buffered,
-// 16-byte slots XOR-swizzled per row).  For every 32-key sub-tile a wave issues, per query and per
-// group of 32 heads, two v_mfma_f32_32x32x64_f8f6f4 (A = the query's fp8 rows, held in registers
-// for the whole sweep; B = key rows from LDS).  The accumulator layout puts one key per lane and 16
-// heads per register file column, so the weighted ReLU-sum over heads is 2 VALU ops per element
-// inside a lane plus one exchange between the two half-waves.  Both the MFMA pipe and the VALU
-// epilogue do 1 operation per (head, key) element at roughly equal cost; the kernel is bound by
-// whichever of the two is busier, never by HBM (q8/k8 are read once, logits written once).
+// One workgroup owns 8 consecutive queries, one per wave (512 threads; at 122 registers per lane
+// four waves share a SIMD), and streams the keys its queries can see through LDS in tiles of 128
+// rows (global_load_lds, double buffered, 16-byte slots XOR-swizzled per row).  For every 32-key
+// sub-tile a wave issues, per group of 32 heads, two v_mfma_f32_32x32x64_f8f6f4 (A = the query's fp8
+// rows, held in registers for the whole sweep; B = key rows from LDS).  The accumulator layout puts
+// one key per lane and 16 heads per register file column, so the weighted ReLU-sum over heads is 2
+// VALU ops per element inside a lane plus one exchange between the two half-waves.  Per sub-tile
+// that is 4 MFMAs of 64 cycles against about 77 VALU issues of 4 cycles: the VALU port is the busier
+// of the two, and the matrix pipe of one wave overlaps the epilogue of the others, not its own -
+// hence the small register footprint and the high occupancy.  HBM is far from binding (q8 / k8 are
+// read once, logits written once).
 #include "dsa_common.h"
 
 namespace {

@@ -1,11 +1,15 @@
 // Per-row top-k selection (radix select with the candidate histograms in LDS) for gfx950.
 //
-// One workgroup per row.  The row's window is read from HBM exactly once into LDS as
-// order-preserving 32-bit keys; three histogram passes (12 + 10 + 10 bits, most significant first)
-// locate the k-th largest key exactly, a prefix-sum compaction then emits every key above it plus
-// the first ties in ascending column order, so the result is deterministic.  An optional bitonic
-// sort in LDS orders the K outputs by descending score.  HBM-bound by design: 4 bytes read per
-// candidate, 8 bytes written per output slot; everything else stays in LDS.
+// One workgroup per row.  General path: the row's window is read once into LDS as order-preserving
+// 32-bit keys (or re-read from global memory when it does not fit); three histogram passes
+// (12 + 10 + 10 bits, most significant first) locate the k-th largest key exactly, a prefix-sum
+// compaction then emits every key above it plus the first ties in ascending column order, so the
+// result is deterministic; an optional sorting network orders the K outputs by descending score.
+// Sorted rows whose values spread over a range take a single sweep instead (linear_select_sort*):
+// a histogram over equal-width value bins, a counting-sort scatter and a rank inside each bin; rows
+// of up to 8192 columns are held in registers for it, which leaves room for four workgroups per
+// compute unit.  HBM-bound by design (4 bytes read per candidate, 8 bytes written per output slot);
+// in practice the LDS atomics of the histogram and the scatter set the pace.
 #include "dsa_common.h"
 
 namespace {
