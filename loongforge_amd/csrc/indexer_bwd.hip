@@ -8,12 +8,14 @@
 // One 256-thread workgroup per query; the four waves each take 32 of the 128 slots of a tile.
 //   r        fp8 MFMA (exact products, as in the forward), one key per lane, heads down the registers
 //   d_k8 row bf16 MFMA  row^T[d, key] = Q^T[d, head] . E[head, key];  E = the r-accumulator layout,
-//            Q^T resident in accumulation registers; the fp32 row goes to a pair buffer at the position
-//            of a key-sorted order and a second kernel sums every key's rows in ascending query order
+//            Q^T resident in accumulation registers; the row, rounded to bf16, goes to a pair buffer at
+//            the position of a key-sorted order and a second kernel sums every key's rows in fp32 in
+//            ascending query order
 //   d_q8     bf16 MFMA  dq^T[d, head] += K^T[d, key] . E^T[key, head], both operands by LDS transpose
 //            reads (the wave's key rows converted to bf16, and E written back to LDS)
-// E is carried as a bf16 pair (hi + lo), so the bf16 products lose nothing visible in fp32; q8 and
-// k8 are exact in bf16.  No floating-point atomics: every sum has a fixed order.
+// For d_q8 E is carried as a bf16 pair (hi + lo), so the bf16 products lose nothing visible in fp32
+// (q8 and k8 are exact in bf16); the d_k8 rows use the hi part alone, as they are rounded to bf16
+// anyway.  No floating-point atomics: every sum has a fixed order.
 #include "dsa_common.h"
 #include "order.h"
 
