@@ -62,6 +62,17 @@ __device__ __forceinline__ void mfma_chain_done(f32x16& acc) {
 // true row maximum with an extra sweep of S^T over all tiles.
 constexpr unsigned LSE_REDO_MARK = 0x7fc0d5a0u;
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned cvt_pk_bf16(float lo, float hi) {    // one v_cvt_pk_bf16_f32
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
+// v_permlane32_swap: the upper half-wave of a trades places with the lower half-wave of b
+__device__ __forceinline__ void swap_halves(unsigned& a, unsigned& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+
 template <int STAGES, int POUT, bool EXACT>   // POUT: 0 none, 1 bf16, 2 f32
 __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
@@ -258,15 +269,28 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
     f32x16 sacc;
     qk_tile(tb, mask, sacc);
     if (POUT != 0 && head_ok && tile * BI >= p_skip) {
-      const size_t pbase = ((size_t)qi * H + h) * (K - p_skip) + (size_t)(tile * BI - p_skip) + 4 * g;
+      const size_t prow = ((size_t)qi * H + h) * (K - p_skip) + (size_t)(tile * BI - p_skip);
+      if (POUT == 2) {
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        if (POUT == 2) {
+        for (int j = 0; j < 4; j++) {
           f32x4 v = {sacc[4 * j], sacc[4 * j + 1], sacc[4 * j + 2], sacc[4 * j + 3]};
-          *(f32x4*)((float*)p_out + pbase + 8 * j) = v;
-        } else {
-          uint2 v = make_uint2(pack_bf16x2(sacc[4 * j], sacc[4 * j + 1]), pack_bf16x2(sacc[4 * j + 2], sacc[4 * j + 3]));
-          *(uint2*)((unsigned short*)p_out + pbase + 8 * j) = v;
+          *(f32x4*)((float*)p_out + prow + 4 * g + 8 * j) = v;
+        }
+      } else {
+        // A lane holds keys 8j + 4g .. +3 of its head (j = 0..3): 8-byte pieces.  The two half-waves
+        // trade pieces so that each lane ends up with 8 consecutive keys, twice: 16-byte stores.
+        unsigned pc[4][2];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          pc[j][0] = cvt_pk_bf16(sacc[4 * j], sacc[4 * j + 1]);
+          pc[j][1] = cvt_pk_bf16(sacc[4 * j + 2], sacc[4 * j + 3]);
+        }
+#pragma unroll
+        for (int jj = 0; jj < 4; jj += 2) {
+          // afterwards (pc[jj], pc[jj + 1]) are keys 8 (jj + g) .. +7
+          swap_halves(pc[jj][0], pc[jj + 1][0]);
+          swap_halves(pc[jj][1], pc[jj + 1][1]);
+          *(uint4*)((unsigned short*)p_out + prow + 8 * (jj + g)) = make_uint4(pc[jj][0], pc[jj][1], pc[jj + 1][0], pc[jj + 1][1]);
         }
       }
     }
