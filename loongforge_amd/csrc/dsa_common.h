@@ -39,6 +39,13 @@ __device__ __forceinline__ unsigned short f32_to_bf16_bits(float f) {   // round
 __device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
   return (unsigned)f32_to_bf16_bits(lo) | ((unsigned)f32_to_bf16_bits(hi) << 16);
 }
+// the same rounding in one instruction (v_cvt_pk_bf16_f32)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned cvt_pk_bf16(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
 // s_waitcnt with only the vector-memory counter constrained (gfx9 encoding).
 #define DSA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 0xf) | (((n) >> 4) << 14)) | (0x7 << 4) | (0xf << 8))
 

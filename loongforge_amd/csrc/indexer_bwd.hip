@@ -25,12 +25,6 @@ constexpr int D = 128;
 constexpr int TK = 128;                 // slots per tile
 constexpr int TILE_BYTES = TK * D;      // fp8 key rows
 constexpr int RED_STRIDE = 132;         // floats per head row of the cross-wave reduction buffer
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ unsigned cvt_pk_bf16(float lo, float hi) {    // one v_cvt_pk_bf16_f32
-  const f32x2_t v = {lo, hi};
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
-}
 constexpr int STRIP_STRIDE = 136;       // bytes per key row of the d_k transpose strip (two d-tiles of 64 bytes + bank spread)
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));

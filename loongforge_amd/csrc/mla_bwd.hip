@@ -333,7 +333,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
       unsigned short* op = (unsigned short*)dq + ((size_t)qi * H + h) * DQK + 32 * dt + 4 * g;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        uint2 w = make_uint2(pack_bf16x2(acc[u][4 * j], acc[u][4 * j + 1]), pack_bf16x2(acc[u][4 * j + 2], acc[u][4 * j + 3]));
+        uint2 w = make_uint2(cvt_pk_bf16(acc[u][4 * j], acc[u][4 * j + 1]), cvt_pk_bf16(acc[u][4 * j + 2], acc[u][4 * j + 3]));
         *(uint2*)(op + 8 * j) = w;
       }
     }
@@ -357,13 +357,6 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
 constexpr int DKV_COEF_STAGES = 3;           // coefficient tiles in the LDS ring
 constexpr int DKV_STRIP_STRIDE = 80;         // bytes per row of the wave-private transpose strip
 constexpr int DKV_STRIP_BYTES = BI * DKV_STRIP_STRIDE;
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ unsigned cvt_pk_bf16(float lo, float hi) {
-  const f32x2_t v = {lo, hi};
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
-}
 
 // NC = column tiles of this wave (5 for waves 0 and 1, else 4).
 template <int NC>

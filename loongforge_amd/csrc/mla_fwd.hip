@@ -62,12 +62,6 @@ __device__ __forceinline__ void mfma_chain_done(f32x16& acc) {
 // true row maximum with an extra sweep of S^T over all tiles.
 constexpr unsigned LSE_REDO_MARK = 0x7fc0d5a0u;
 
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ unsigned cvt_pk_bf16(float lo, float hi) {    // one v_cvt_pk_bf16_f32
-  const f32x2_t v = {lo, hi};
-  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
-}
 // v_permlane32_swap: the upper half-wave of a trades places with the lower half-wave of b
 __device__ __forceinline__ void swap_halves(unsigned& a, unsigned& b) {
   asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
@@ -377,8 +371,8 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
     for (int dt = 0; dt < DTILES; dt++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        uint2 v = make_uint2(pack_bf16x2(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
-                             pack_bf16x2(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv));
+        uint2 v = make_uint2(cvt_pk_bf16(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
+                             cvt_pk_bf16(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv));
         *(uint2*)(op + 32 * dt + 8 * j) = v;
       }
   }
