@@ -46,6 +46,28 @@ __device__ __forceinline__ unsigned cvt_pk_bf16(float lo, float hi) {
   const f32x2_t v = {lo, hi};
   return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
 }
+// v_permlane32_swap: the upper half-wave of a trades places with the lower half-wave of b.
+__device__ __forceinline__ void swap_halves(unsigned& a, unsigned& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+// A 32 x 32 MFMA accumulator gives lane (r, g = lane / 32) the elements 8j + 4g .. +3 (j = 0..3) of row
+// segment r: four 8-byte pieces once rounded to bf16.  The two half-waves trade pieces so that the lane
+// ends up with elements 8 (jj + g) .. +7 for jj = 0 and jj = 2: two 16-byte values, o[0] and o[1].
+// Every lane of the wave must take part.
+__device__ __forceinline__ void acc_row_to_16B(const f32x16& acc, float scale, uint4 (&o)[2]) {
+  unsigned pc[4][2];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    pc[j][0] = cvt_pk_bf16(acc[4 * j] * scale, acc[4 * j + 1] * scale);
+    pc[j][1] = cvt_pk_bf16(acc[4 * j + 2] * scale, acc[4 * j + 3] * scale);
+  }
+#pragma unroll
+  for (int jj = 0; jj < 4; jj += 2) {
+    swap_halves(pc[jj][0], pc[jj + 1][0]);
+    swap_halves(pc[jj][1], pc[jj + 1][1]);
+    o[jj >> 1] = make_uint4(pc[jj][0], pc[jj][1], pc[jj + 1][0], pc[jj + 1][1]);
+  }
+}
 // s_waitcnt with only the vector-memory counter constrained (gfx9 encoding).
 #define DSA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 0xf) | (((n) >> 4) << 14)) | (0x7 << 4) | (0xf << 8))
 

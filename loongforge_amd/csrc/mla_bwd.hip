@@ -329,13 +329,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
     const int dt = u < 16 ? 4 * wave + (u >> 2) : 16 + (wave >> 1);
     const int hg = u < 16 ? (u & 3) : hg_last + (u - 16);
     const int h = hg * 32 + r;
-    if (h < H) {
-      unsigned short* op = (unsigned short*)dq + ((size_t)qi * H + h) * DQK + 32 * dt + 4 * g;
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        uint2 w = make_uint2(cvt_pk_bf16(acc[u][4 * j], acc[u][4 * j + 1]), cvt_pk_bf16(acc[u][4 * j + 2], acc[u][4 * j + 3]));
-        *(uint2*)(op + 8 * j) = w;
-      }
+    if (h < H) {                               // the same for all lanes of a wave (H is a multiple of 32)
+      unsigned short* op = (unsigned short*)dq + ((size_t)qi * H + h) * DQK + 32 * dt + 8 * g;
+      uint4 o[2];
+      acc_row_to_16B(acc[u], 1.0f, o);
+      *(uint4*)op = o[0];
+      *(uint4*)(op + 16) = o[1];
     }
   }
 }

@@ -62,11 +62,6 @@ __device__ __forceinline__ void mfma_chain_done(f32x16& acc) {
 // true row maximum with an extra sweep of S^T over all tiles.
 constexpr unsigned LSE_REDO_MARK = 0x7fc0d5a0u;
 
-// v_permlane32_swap: the upper half-wave of a trades places with the lower half-wave of b
-__device__ __forceinline__ void swap_halves(unsigned& a, unsigned& b) {
-  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-}
-
 template <int STAGES, int POUT, bool EXACT>   // POUT: 0 none, 1 bf16, 2 f32
 __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
@@ -273,19 +268,10 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
       } else {
         // A lane holds keys 8j + 4g .. +3 of its head (j = 0..3): 8-byte pieces.  The two half-waves
         // trade pieces so that each lane ends up with 8 consecutive keys, twice: 16-byte stores.
-        unsigned pc[4][2];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          pc[j][0] = cvt_pk_bf16(sacc[4 * j], sacc[4 * j + 1]);
-          pc[j][1] = cvt_pk_bf16(sacc[4 * j + 2], sacc[4 * j + 3]);
-        }
-#pragma unroll
-        for (int jj = 0; jj < 4; jj += 2) {
-          // afterwards (pc[jj], pc[jj + 1]) are keys 8 (jj + g) .. +7
-          swap_halves(pc[jj][0], pc[jj + 1][0]);
-          swap_halves(pc[jj][1], pc[jj + 1][1]);
-          *(uint4*)((unsigned short*)p_out + prow + 8 * (jj + g)) = make_uint4(pc[jj][0], pc[jj][1], pc[jj + 1][0], pc[jj + 1][1]);
-        }
+        uint4 o[2];
+        acc_row_to_16B(sacc, 1.0f, o);
+        *(uint4*)((unsigned short*)p_out + prow + 8 * g) = o[0];
+        *(uint4*)((unsigned short*)p_out + prow + 16 + 8 * g) = o[1];
       }
     }
 
@@ -366,15 +352,14 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
   const float inv = l_tot > 0.f ? o_scale / l_tot : 0.f;
   if (head_ok) {
     if (g == 0) lse[(size_t)qi * H + h] = l_tot > 0.f ? (m_ref + log2f(l_tot)) * 0.6931471805599453f : INFINITY;
-    unsigned short* op = (unsigned short*)out + ((size_t)qi * H + h) * DV + 4 * g;
+    unsigned short* op = (unsigned short*)out + ((size_t)qi * H + h) * DV + 8 * g;
 #pragma unroll
-    for (int dt = 0; dt < DTILES; dt++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        uint2 v = make_uint2(cvt_pk_bf16(oacc[dt][4 * j] * inv, oacc[dt][4 * j + 1] * inv),
-                             cvt_pk_bf16(oacc[dt][4 * j + 2] * inv, oacc[dt][4 * j + 3] * inv));
-        *(uint2*)(op + 32 * dt + 8 * j) = v;
-      }
+    for (int dt = 0; dt < DTILES; dt++) {
+      uint4 o[2];
+      acc_row_to_16B(oacc[dt], inv, o);       // head_ok is the same for all lanes of a wave
+      *(uint4*)(op + 32 * dt) = o[0];
+      *(uint4*)(op + 32 * dt + 16) = o[1];
+    }
   }
 }
 
