@@ -94,13 +94,22 @@ __global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
     const bf16x8* op = (const bf16x8*)(out + hrow * DV) + g;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) qreg[ks] = qp[2 * ks];
+#pragma unroll
+    for (int ks = 0; ks < VSTEPS; ks++) doreg[ks] = dp[2 * ks];
+    // delta = rowsum(O . dO): the O rows come in four batches of eight loads, so that a batch costs
+    // one round trip instead of eight (the fences keep the loads of a batch together)
     float part = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < VSTEPS; ks++) {
-      doreg[ks] = dp[2 * ks];
-      const bf16x8 o = op[2 * ks];
+    for (int b = 0; b < VSTEPS / 8; b++) {
+      bf16x8 o[8];
 #pragma unroll
-      for (int e = 0; e < 8; e++) part = fmaf((float)o[e], (float)doreg[ks][e], part);
+      for (int i = 0; i < 8; i++) o[i] = op[2 * (8 * b + i)];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) part = fmaf((float)o[i][e], (float)doreg[8 * b + i][e], part);
+      __builtin_amdgcn_sched_barrier(0);
     }
     part += __shfl_xor(part, 32, 64);
     if (g == 0) {
