@@ -163,6 +163,7 @@ def main():
     lg = ops.indexer_logits(q8, wsd, k8, ksc, ks, ke)          # untimed first call
     ops.topk(lg, K, ks, ke)
     torch.cuda.synchronize()
+    del lg                                                     # the timed call reuses this block: no allocation inside the timing
     e0, e1, e2 = ev(), ev(), ev()
     e0.record()
     lg = ops.indexer_logits(q8, wsd, k8, ksc, ks, ke)
@@ -216,6 +217,26 @@ def main():
     t_rope = e0.elapsed_time(e1) / 5
     del qc, qpe
 
+    # what plain data movers with the traffic shape of the two bandwidth-bound backward passes reach:
+    # as many 1152-byte rows as the dKV pass writes, at scattered positions, beside a streaming read
+    # of 0.6 x that size (P, dS, Q, dO); and a streaming read of the rows (the ordered sum).  Source
+    # and destination are carved out of the backward's workspace, which is scratch between calls.
+    rows_per_wg = int(pairs // S) // 4 * 4
+    row_bytes = S * rows_per_wg * 1152
+    steps4 = rows_per_wg // 4
+    src_bytes = S * (steps4 // 5 * 3 + min(steps4 % 5, 3)) * 4608
+    mover = None
+    if row_bytes + src_bytes + 256 <= wsb:
+        src_ptr = ws.data_ptr() + (row_bytes + 255) // 256 * 256
+        sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+        t_rows, _ = timed(lambda: _lib.check(lib.dsa_probe_hbm_rows(src_ptr, ws.data_ptr(), S, rows_per_wg, 3, 1, stream),
+                                             "probe rows"))
+        t_read, _ = timed(lambda: _lib.check(lib.dsa_probe_hbm_read(ws.data_ptr(), row_bytes, sink.data_ptr(), stream),
+                                             "probe read"))
+        mover = {"rows_written_scattered_plus_stream_read_gbps": round((row_bytes + src_bytes) / (t_rows * 1e-3) / 1e9, 1),
+                 "stream_read_gbps": round(row_bytes / (t_read * 1e-3) / 1e9, 1),
+                 "note": "plain movers with the byte counts and access shape of bwd_dkv_kernel and bwd_reduce_kernel"}
+
     mla_tflops = (flops_fwd + flops_bwd) / ((t_fwd + t_bwd) * 1e-3) / 1e12
     # ---- roofline of the longest-running kernel of the step ---------------------------------------
     # Per kernel: algorithmic flops and algorithmic HBM bytes of one launch.  Gathered key rows are
@@ -248,6 +269,10 @@ def main():
     roofline["avg_launch_ms"] = round(t_dom, 3)
     roofline["algorithmic_bytes"] = b_dom
     roofline["algorithmic_flops"] = f_dom
+    if mover is not None and roofline["bound"] == "hbm":
+        # the same launch against the measured rate of a plain mover of its traffic shape
+        ref = mover["rows_written_scattered_plus_stream_read_gbps" if name.startswith("bwd_dkv") else "stream_read_gbps"]
+        roofline["frac_of_plain_mover"] = round(roofline["achieved"] / ref, 4)
     if args.copy_calibration:
         # a plain 1 GiB device copy: the known-size kernel the HBM counters are scaled by
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -293,6 +318,7 @@ def main():
         "rope_permute_cat_ms": round(t_rope, 3),
         "rope_permute_cat_gbps": round(4.0 * S * H * DQK / (t_rope * 1e-3) / 1e9, 1),
         "wall_s_per_step": round(wall / n, 4),
+        "hbm_plain_mover": mover,
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:

@@ -219,6 +219,22 @@ int dsa_rope_headsum_inverse(const void* grad, int64_t g_tok, int64_t g_head, vo
                              const int32_t* positions, int batch, int tokens, int heads, int in_pairing,
                              void* stream);
 
+/*
+ * Measurement aids; no counterpart in the reference.  Plain data movers with the traffic shape of
+ * the two bandwidth-bound backward passes, so that a benchmark can quote those passes against what
+ * the memory system gives a kernel that does nothing else.
+ *
+ * dsa_probe_hbm_rows: `workgroups` x `rows_per_workgroup` (a multiple of 4) rows of 1152 bytes are
+ * written to `rows` (at permuted row positions when scatter != 0, in order otherwise) while each
+ * workgroup streams 4608 bytes from `src` on read_fifths (0..5) of every 5 steps of 4 rows; with
+ * n = rows_per_workgroup / 4 steps, src must hold
+ * workgroups * (n / 5 * read_fifths + min(n % 5, read_fifths)) * 4608 bytes.
+ * dsa_probe_hbm_read: streams `bytes` from src; sink16 points at 16 writable bytes.
+ */
+int dsa_probe_hbm_rows(const void* src, void* rows, int workgroups, int rows_per_workgroup, int read_fifths,
+                       int scatter, void* stream);
+int dsa_probe_hbm_read(const void* src, size_t bytes, void* sink16, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
