@@ -625,7 +625,7 @@ __global__ void cast_bf16_kernel(const float* __restrict__ src, unsigned short* 
 struct BwdPlan {
   int chunk;            // queries per pass over the buffers
   int W;                // bitmap words per key
-  size_t off_bitmap, off_prefix, off_count, off_start, off_dst, off_pds, off_rows, off_acc, total;
+  size_t off_bitmap, off_prefix, off_count, off_start, off_dst, off_sorted, off_pds, off_rows, off_acc, total;
 };
 
 size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -640,6 +640,7 @@ BwdPlan layout_plan(int chunk, int Skv, int K) {
   p.off_count = o; o = align_up(o + (size_t)(Skv + 1) * 4);
   p.off_start = o; o = align_up(o + (size_t)(Skv + 1) * 4);
   p.off_dst = o; o = align_up(o + (size_t)chunk * K * 4);
+  p.off_sorted = o; o = align_up(o + (size_t)chunk * K * 4);
   p.off_pds = o; o = align_up(o + (size_t)chunk * (K / BI) * PDS_TILE_BYTES);
   p.off_rows = o; o = align_up(o + ((size_t)chunk * K + 1) * ROW_BYTES);
   p.off_acc = o; o = align_up(o + (size_t)Skv * DQK * 4);
@@ -692,6 +693,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   int* count = (int*)(ws + p.off_count);
   int* start = (int*)(ws + p.off_start);
   int* dstp = (int*)(ws + p.off_dst);
+  int* sorted = (int*)(ws + p.off_sorted);
   unsigned char* pds = ws + p.off_pds;
   unsigned char* rows = ws + p.off_rows;
   float* acc = (float*)(ws + p.off_acc);
@@ -716,17 +718,21 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   for (int q0 = 0; q0 < S; q0 += p.chunk) {
     const int cnt = S - q0 < p.chunk ? S - q0 : p.chunk;
     DSA_MARK(0);
-    order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st);
+    // The passes are free to choose their slot order (P, dS and the dKV rows never leave the workspace):
+    // they walk each query's valid ids in ascending key order, so that the queries in flight on an XCD
+    // gather neighbouring latent rows at the same time.
+    order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st, sorted);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
+    const int* sids = sorted - (size_t)q0 * K;          // indexed by global query, like ids
     DSA_MARK(1);
-    bwd_pds_kernel<4><<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (const __bf16*)out,
+    bwd_pds_kernel<4><<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out,
                                                           (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(P, dS)");
     DSA_MARK(2);
-    bwd_dq_kernel<3><<<dim3(cnt), dim3(256), smemB, st>>>((const __bf16*)kv, ids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start);
+    bwd_dq_kernel<3><<<dim3(cnt), dim3(256), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ)");
     DSA_MARK(3);
-    bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, ids, pds, dstp, rows, q0, cnt,
+    bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, sids, pds, dstp, rows, q0, cnt,
                                                        H, Skv, K, q_start, p.chunk * K);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV rows)");
     DSA_MARK(4);

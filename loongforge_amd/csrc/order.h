@@ -20,8 +20,10 @@ static __global__ void zero_u32_kernel(unsigned* __restrict__ p, size_t n) {
 // masks of 4 such query groups are combined through LDS so that every key receives 32 contiguous
 // bytes.
 static __global__ __launch_bounds__(256) void qmap_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv,
-                                                          int q_start, unsigned* __restrict__ qmap, int Wk) {
-  extern __shared__ unsigned qbits[];        // Wk words
+                                                          int q_start, unsigned* __restrict__ qmap, int Wk,
+                                                          int* __restrict__ sorted) {
+  extern __shared__ unsigned qbits[];        // Wk words; with `sorted`, Wk more for the prefix counts
+  __shared__ int wave_tot[4];
   const int ql = blockIdx.x;
   for (int w = threadIdx.x; w < Wk; w += 256) qbits[w] = 0u;
   __syncthreads();
@@ -35,6 +37,33 @@ static __global__ __launch_bounds__(256) void qmap_kernel(const int* __restrict_
   }
   __syncthreads();
   for (int w = threadIdx.x; w < Wk; w += 256) qmap[(size_t)ql * Wk + w] = qbits[w];
+  if (sorted == nullptr) return;
+  // The query's valid ids in ascending order, -1 after them: id v goes to position (set bits below v).
+  // Thread t counts the words [t * per, (t + 1) * per); an exclusive scan over the threads gives each
+  // thread its base, from which it writes the per-word prefix counts.
+  unsigned* pre = qbits + Wk;
+  const int per = (Wk + 255) / 256;
+  const int w0 = threadIdx.x * per;
+  int mine = 0;
+  for (int w = w0; w < w0 + per && w < Wk; w++) mine += __popc(qbits[w]);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int inc = mine;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) { int n = __shfl_up(inc, o, 64); if (lane >= o) inc += n; }
+  if (lane == 63) wave_tot[wave] = inc;
+  __syncthreads();
+  int base = inc - mine;
+  for (int w = 0; w < wave; w++) base += wave_tot[w];
+  const int total = wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+  for (int w = w0; w < w0 + per && w < Wk; w++) { pre[w] = (unsigned)base; base += __popc(qbits[w]); }
+  __syncthreads();
+  int* row = sorted + (size_t)ql * K;
+  for (int t = threadIdx.x; t < K; t += 256) {
+    const int v = ids[(size_t)(q0 + ql) * K + t];
+    if (v >= 0 && v < Skv && v <= q_start + q0 + ql)
+      row[pre[v >> 5] + __popc(qbits[v >> 5] & ((1u << (v & 31)) - 1u))] = v;
+  }
+  for (int t = total + threadIdx.x; t < K; t += 256) row[t] = -1;
 }
 
 // grid (ceil(cnt / 256), Wk); workgroup = 4 waves = 256 queries of one key word
@@ -123,6 +152,10 @@ static __global__ void rank_kernel(const int* __restrict__ ids, int q0, int cnt,
 
 // Launches the five kernels above for queries [q0, q0 + cnt).  A slot counts when its id v is in
 // [0, Skv) and v <= q_start + (query index); pass a huge q_start to accept every id in range.
+// With `sorted` ([cnt][K] ints) the first kernel also writes every query's valid ids in ascending
+// order (-1 after them) and dst refers to the slots of that list: a caller that is free to choose
+// its slot order uses the list instead of ids, which makes concurrently running queries gather
+// neighbouring key rows at the same time (the rows then hit in the L2 of the XCD).
 // The prefix buffer doubles as the scratch of step (1) (cnt * ceil(Skv / 32) words; it is rewritten by
 // the prefix pass afterwards): size it with prefix_words().
 inline size_t prefix_words(int chunk, int Skv) {
@@ -130,18 +163,21 @@ inline size_t prefix_words(int chunk, int Skv) {
   return (size_t)Skv * W > (size_t)chunk * Wk ? (size_t)Skv * W : (size_t)chunk * Wk;
 }
 inline void build(const int* ids, int q0, int cnt, int K, int Skv, int q_start, unsigned* bitmap, unsigned* prefix,
-                  int* count, int* start, int* dst, int W, hipStream_t st) {
+                  int* count, int* start, int* dst, int W, hipStream_t st, int* sorted = nullptr) {
   const int Wk = (Skv + 31) / 32;
   unsigned* qmap = prefix;
-  if ((size_t)Wk * 4 > 48 * 1024)
-    (void)hipFuncSetAttribute((const void*)qmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Wk * 4);
-  qmap_kernel<<<dim3(cnt), dim3(256), (size_t)Wk * 4, st>>>(ids, q0, cnt, K, Skv, q_start, qmap, Wk);
+  const size_t lds = (size_t)Wk * 4 * (sorted ? 2 : 1);
+  if (lds > 48 * 1024)
+    (void)hipFuncSetAttribute((const void*)qmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  qmap_kernel<<<dim3(cnt), dim3(256), lds, st>>>(ids, q0, cnt, K, Skv, q_start, qmap, Wk, sorted);
   // every word of the bitmap is written (zeros beyond the last query), so no clearing pass is needed
   bm_transpose_kernel<<<dim3((W + 7) / 8, Wk), dim3(256), 0, st>>>(qmap, cnt, Skv, Wk, bitmap, W);
   bm_prefix_kernel<<<dim3((Skv + 3) / 4), dim3(256), 0, st>>>(bitmap, prefix, count, Skv, W);
   key_scan_kernel<<<dim3(1), dim3(1024), 0, st>>>(count, start, Skv);
-  rank_kernel<<<dim3((K + 255) / 256, cnt < 32768 ? cnt : 32768), dim3(256), 0, st>>>(ids, q0, cnt, K, Skv, q_start, bitmap, prefix,
-                                                                                     start, W, dst);
+  // with `sorted` (rows of the block's queries, [cnt][K]) the ranks are those of the sorted slots
+  const int* rank_ids = sorted ? sorted - (size_t)q0 * K : ids;
+  rank_kernel<<<dim3((K + 255) / 256, cnt < 32768 ? cnt : 32768), dim3(256), 0, st>>>(rank_ids, q0, cnt, K, Skv, q_start, bitmap,
+                                                                                     prefix, start, W, dst);
 }
 
 }  // namespace order
