@@ -22,7 +22,7 @@ static __global__ void zero_u32_kernel(unsigned* __restrict__ p, size_t n) {
 static __global__ __launch_bounds__(256) void qmap_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv,
                                                           int q_start, unsigned* __restrict__ qmap, int Wk,
                                                           int* __restrict__ sorted) {
-  extern __shared__ unsigned qbits[];        // Wk words; with `sorted`, Wk more for the prefix counts
+  extern __shared__ unsigned qbits[];        // Wk words; with `sorted`, Wk more for the prefix counts and K for the list
   __shared__ int wave_tot[4];
   const int ql = blockIdx.x;
   for (int w = threadIdx.x; w < Wk; w += 256) qbits[w] = 0u;
@@ -57,13 +57,16 @@ static __global__ __launch_bounds__(256) void qmap_kernel(const int* __restrict_
   const int total = wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
   for (int w = w0; w < w0 + per && w < Wk; w++) { pre[w] = (unsigned)base; base += __popc(qbits[w]); }
   __syncthreads();
-  int* row = sorted + (size_t)ql * K;
+  int* list = (int*)(pre + Wk);              // K ints: the list is put together in LDS and written out in order
+  for (int t = total + threadIdx.x; t < K; t += 256) list[t] = -1;
   for (int t = threadIdx.x; t < K; t += 256) {
     const int v = ids[(size_t)(q0 + ql) * K + t];
     if (v >= 0 && v < Skv && v <= q_start + q0 + ql)
-      row[pre[v >> 5] + __popc(qbits[v >> 5] & ((1u << (v & 31)) - 1u))] = v;
+      list[pre[v >> 5] + __popc(qbits[v >> 5] & ((1u << (v & 31)) - 1u))] = v;
   }
-  for (int t = total + threadIdx.x; t < K; t += 256) row[t] = -1;
+  __syncthreads();
+  int* row = sorted + (size_t)ql * K;
+  for (int t = threadIdx.x; t < K; t += 256) row[t] = list[t];
 }
 
 // grid (ceil(cnt / 256), Wk); workgroup = 4 waves = 256 queries of one key word
@@ -166,7 +169,7 @@ inline void build(const int* ids, int q0, int cnt, int K, int Skv, int q_start, 
                   int* count, int* start, int* dst, int W, hipStream_t st, int* sorted = nullptr) {
   const int Wk = (Skv + 31) / 32;
   unsigned* qmap = prefix;
-  const size_t lds = (size_t)Wk * 4 * (sorted ? 2 : 1);
+  const size_t lds = (size_t)Wk * 4 * (sorted ? 2 : 1) + (sorted ? (size_t)K * 4 : 0);
   if (lds > 48 * 1024)
     (void)hipFuncSetAttribute((const void*)qmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   qmap_kernel<<<dim3(cnt), dim3(256), lds, st>>>(ids, q0, cnt, K, Skv, q_start, qmap, Wk, sorted);
