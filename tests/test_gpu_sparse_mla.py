@@ -129,6 +129,27 @@ def test_backward_against_oracle_and_deterministic(gpu, S, H, K, q_start, skv, s
     assert torch.equal(dq, dq2) and torch.equal(dkv, dkv2)          # bit-identical
 
 
+def test_backward_does_not_depend_on_the_slot_order(gpu):
+    """The backward walks each query's ids in ascending key order whatever order they arrive in, so
+    permuting the slots (independently per query) and scattering unused slots between the used ones
+    gives bit-identical gradients."""
+    from loongforge_amd import ops
+
+    S, K = 150, 128
+    inp = O.make_mla_inputs(S, 128, 96, seed=9)                       # 96 used slots ...
+    idx = torch.cat([inp.idx, torch.full((S, K - 96), -1, dtype=torch.int32)], dim=1)
+    g = torch.Generator().manual_seed(3)
+    shuffled = torch.stack([idx[i][torch.randperm(K, generator=g)] for i in range(S)])      # ... anywhere among 128
+    q, kv, do = inp.q.to(gpu), inp.kv.to(gpu), inp.dout.to(gpu)
+    out, lse, _ = ops.sparse_mla_fwd(q, kv, idx.to(gpu), 0, inp.sm_scale)
+    dq1, dkv1 = ops.sparse_mla_bwd(q, kv, out, do, idx.to(gpu), lse, 0, inp.sm_scale)
+    dq2, dkv2 = ops.sparse_mla_bwd(q, kv, out, do, shuffled.to(gpu), lse, 0, inp.sm_scale)
+    assert torch.equal(dq1, dq2) and torch.equal(dkv1, dkv2)
+    rdq, rdkv = O.sparse_mla_bwd(inp.q, inp.kv, inp.idx, inp.dout, 0, inp.sm_scale, 512)
+    assert_close(dq2, rdq, "dq", scale_aware=True)
+    assert_close(dkv2, rdkv, "dkv", scale_aware=True)
+
+
 def test_forward_and_backward_with_attention_sink(gpu):
     from loongforge_amd import ops
 
