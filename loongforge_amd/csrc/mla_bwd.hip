@@ -198,19 +198,25 @@ __global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
 // ---------------------------------------------------------------------------------------------
 // dQ^T[d, head] += KV^T[d, key] . dS^T[key, head] per 32-key tile.  Both operands are LDS transpose
 // reads: of the gathered key tile (18 d-tiles) and of the tile's dS block copied verbatim from the
-// pass-A buffer.  The 72 accumulator tiles (18 d-tiles x 4 head groups) are split over the waves
-// by d: wave w owns d-tiles 4w .. 4w+3 for all four head groups, plus d-tile 16 + w/2 for head
-// groups 2(w%2), 2(w%2)+1 - 18 tiles (288 registers: 256 accumulation + 32 architectural) and 36
-// MFMAs per wave and tile.  A key-tile operand read from LDS then feeds up to four MFMAs, and the
-// eight dS operands of a tile are read once per wave: 72 KB of LDS reads per tile instead of the
-// 152 KB of a split by heads.
+// pass-A buffer.  Eight waves share the 72 accumulator tiles (18 d-tiles x 4 head groups): wave
+// (w, hh) = (wave % 4, wave / 4) owns d-tiles 4w .. 4w+3 for the head groups 2hh, 2hh+1, plus d-tile
+// 16 + w/2 for head group 2hh + w%2 - 9 tiles (144 accumulator registers) and 18 MFMAs per wave and
+// tile.  (The wave keeps its two head groups in the order hgs[0] = 2hh + w%2, hgs[1] = the other one,
+// so that the ninth tile always uses operand 0: a run-time choice between two MFMAs would make the
+// compiler copy the accumulator between registers right after an MFMA it cannot see into.)  At under 256 registers per lane two waves share a SIMD, so that while one of them is held
+// up issuing its part of the next tile's transfers (the address unit takes them at 64 B/clk for the
+// whole compute unit) the other one keeps the matrix pipe busy; with four waves of 288 accumulator
+// registers nothing filled that gap.  A key-tile operand read from LDS feeds two MFMAs: 112 KB of
+// LDS reads per tile, below the 147 KB the matrix pipe's time allows.
 template <int STAGES>
-__global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
+__global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
     const __bf16* __restrict__ kv, const int* __restrict__ ids, const unsigned char* __restrict__ pds,
     __bf16* __restrict__ dq, int q0, int cnt, int H, int Skv, int K, int q_start) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int STAGE_BYTES = TILE_BYTES + PDS_KIND_BYTES;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int w = wave & 3, hh = wave >> 2;
   const int r = lane & 31, g = lane >> 5;
   const int ql = cnt - 1 - (int)blockIdx.x;
   const int qi = q0 + ql;
@@ -219,6 +225,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
   unsigned* tmask = (unsigned*)(idx_s + K);
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
+  // (the helper is written for four waves; the other four repeat part of its work with equal results)
   const int ntiles = stage_ids(ids, qi, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
 
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
@@ -238,13 +245,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
         ds_off[s][t] = (unsigned)(TILE_BYTES + key * 64 + (blk & 1) * 32 + (qq & 1) * 16 + (qq >> 1) * 8);
       }
   }
-  // piece P of the LDS order comes from piece src_piece(P) of the HBM order
+  // piece P of the LDS order comes from piece src_piece(P) of the HBM order; thread P moves piece P
   auto src_piece = [](int P) { return (P >> 7) * 128 + ((P >> 1) & 1) * 64 + (P & 1) * 32 + ((P >> 2) & 31); };
-  const unsigned ds_src0 = (unsigned)src_piece(tid) * 16u, ds_src1 = (unsigned)src_piece(tid + 256) * 16u;
-  // key-tile operand offsets of this wave's d-tiles: i = 0..3 -> d-tile 4*wave + i, i = 4 -> 16 + wave/2
-  const unsigned grp_main = (unsigned)(2 * wave) * GRP_BYTES;          // (4w + i) >> 1 = 2w + (i >> 1)
+  const unsigned ds_src = (unsigned)src_piece(tid) * 16u;
+  // key-tile operand offsets of this wave's d-tiles: i = 0..3 -> d-tile 4*w + i, i = 4 -> 16 + w/2
+  const unsigned grp_main = (unsigned)(2 * w) * GRP_BYTES;             // (4w + i) >> 1 = 2w + (i >> 1)
   const unsigned grp_last = (unsigned)(8 * GRP_BYTES);                 // (16 + w/2) >> 1 = 8
-  const int par_last = (wave >> 1) & 1;
+  const int par_last = (w >> 1) & 1;
   unsigned tr_last[2][2];
   {
     // same formula as LaneOffsets::tr_off, with the parity of the d-tile known only at run time
@@ -258,23 +265,37 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
         tr_last[s][t] = (unsigned)(key * 128 + (((4 * par_last + cl) ^ swz(key)) << 4) + half * 8) + grp_last;
       }
   }
-  const int hg_last = 2 * (wave & 1);
+  // Transfers of a tile: the key rows as nine 128-byte groups per row, thread (key, sub) of either half of
+  // the workgroup moving 16 bytes of a group (waves 0-3 take groups 0-4, waves 4-7 groups 5-8), and the
+  // 8 KB dS block, 16 bytes per thread.
+  const int per_issue = hh ? 5 : 6;          // transfers per wave and tile
   auto issue = [&](int n) {
     const int tile = tlist[n];
     const unsigned sb = lds0 + (unsigned)((n % STAGES) * STAGE_BYTES);
-    gather_tile(kv, idx_s, tile, sb);
-    const unsigned lb = __builtin_amdgcn_readfirstlane(sb + (unsigned)(TILE_BYTES + wave * 1024));
+    const int gkey = (tid & 255) >> 3, gsub = tid & 7;
+    int kid = idx_s[tile * BI + gkey];
+    kid = kid < 0 ? 0 : kid;
+    const unsigned goff = (unsigned)kid * (DQK * 2) + (unsigned)((gsub ^ swz(gkey)) * 16);
+    const unsigned lb = __builtin_amdgcn_readfirstlane(sb + (unsigned)(w * 1024));
+    if (hh == 0) {
+#pragma unroll
+      for (int grp = 0; grp < 5; grp++) dma16(lb + grp * GRP_BYTES, goff + grp * 128, kv);
+    } else {
+#pragma unroll
+      for (int grp = 5; grp < 9; grp++) dma16(lb + grp * GRP_BYTES, goff + grp * 128, kv);
+    }
+    const unsigned lbd = __builtin_amdgcn_readfirstlane(sb + (unsigned)(TILE_BYTES + wave * 1024));
     const unsigned char* src = uniform_ptr(pds + ((size_t)ql * NT + tile) * PDS_TILE_BYTES);     // dS half
-    dma16(lb, ds_src0, src);
-    dma16(lb + 4096, ds_src1, src);
+    dma16(lbd, ds_src, src);
   };
 
-  f32x16 acc[18];     // u < 16: d-tile 4*wave + u/4, head group u%4; u = 16, 17: d-tile 16 + wave/2, head group hg_last + u - 16
+  const int hg0 = 2 * hh + (w & 1), hg1 = 2 * hh + 1 - (w & 1);       // the wave's head groups, in its operand order
+  f32x16 acc[9];      // u < 8: d-tile 4w + u/2, head group hg0 (u even) or hg1 (u odd); u = 8: d-tile 16 + w/2, head group hg0
 #pragma unroll
-  for (int u = 0; u < 18; u++) {
+  for (int u = 0; u < 9; u++) {
 #pragma unroll
     for (int e = 0; e < 16; e++) acc[u][e] = 0.f;
-    if (u < 16) asm volatile("" : "+a"(acc[u])); else asm volatile("" : "+v"(acc[u]));
+    if (u < 8) asm volatile("" : "+a"(acc[u])); else asm volatile("" : "+v"(acc[u]));
   }
   typedef short i16x8 __attribute__((ext_vector_type(8)));
   auto tr_pair = [&](const unsigned char* p0, const unsigned char* p1) {
@@ -284,16 +305,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
   };
   for (int n = 0; n < STAGES - 1 && n < ntiles; n++) issue(n);
   for (int n = 0; n < ntiles; n++) {
-    wait_vmcnt_le(11 * min(STAGES - 2, ntiles - 1 - n));
+    wait_vmcnt_le(per_issue * min(STAGES - 2, ntiles - 1 - n));
     __syncthreads();
     if (n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
     const unsigned char* tb = smem + (n % STAGES) * STAGE_BYTES;
-    // the eight dS operands of the tile: [head group][k-step]
-    bf16x8 bds[4][2];
+    // the four dS operands of the wave's two head groups: [hg0 or hg1][k-step]
+    bf16x8 bds[2][2];
 #pragma unroll
-    for (int hg = 0; hg < 4; hg++)
+    for (int j = 0; j < 2; j++)
 #pragma unroll
-      for (int s = 0; s < 2; s++) bds[hg][s] = tr_pair(tb + hg * 2048 + ds_off[s][0], tb + hg * 2048 + ds_off[s][1]);
+      for (int s = 0; s < 2; s++)
+        bds[j][s] = tr_pair(tb + (j ? hg1 : hg0) * 2048 + ds_off[s][0], tb + (j ? hg1 : hg0) * 2048 + ds_off[s][1]);
     // key-tile operands, one d-tile ahead
     bf16x8 a[2][2];
 #pragma unroll
@@ -316,16 +338,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
       for (int s = 0; s < 2; s++) {
         if (i < 4) {
 #pragma unroll
-          for (int hg = 0; hg < 4; hg++) mfma_a_vv(acc[4 * i + hg], a[i & 1][s], bds[hg][s]);
+          for (int j = 0; j < 2; j++) mfma_a_vv(acc[2 * i + j], a[i & 1][s], bds[j][s]);
         } else {
-          // head groups hg_last, hg_last + 1 (a branch, so that no register array is indexed at run time)
-          if (hg_last) {
-            mfma_v_vv(acc[16], a[i & 1][s], bds[2][s]);
-            mfma_v_vv(acc[17], a[i & 1][s], bds[3][s]);
-          } else {
-            mfma_v_vv(acc[16], a[i & 1][s], bds[0][s]);
-            mfma_v_vv(acc[17], a[i & 1][s], bds[1][s]);
-          }
+          mfma_v_vv(acc[8], a[i & 1][s], bds[0][s]);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -333,10 +348,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(
   }
   // ---- write dQ: accumulator e of a lane is d = 32*dt + 8*(e/4) + 4*g + (e%4), head = 32*hg + r ----
 #pragma unroll
-  for (int u = 0; u < 18; u++) {
-    if (u < 16) mfma_done_a(acc[u]); else mfma_done_v(acc[u]);
-    const int dt = u < 16 ? 4 * wave + (u >> 2) : 16 + (wave >> 1);
-    const int hg = u < 16 ? (u & 3) : hg_last + (u - 16);
+  for (int u = 0; u < 9; u++) {
+    if (u < 8) mfma_done_a(acc[u]); else mfma_done_v(acc[u]);
+    const int dt = u < 8 ? 4 * w + (u >> 1) : 16 + (w >> 1);
+    const int hg = (u & 1) ? hg1 : hg0;
     const int h = hg * 32 + r;
     if (h < H) {                               // the same for all lanes of a wave (H is a multiple of 32)
       unsigned short* op = (unsigned short*)dq + ((size_t)qi * H + h) * DQK + 32 * dt + 8 * g;
@@ -729,7 +744,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
                                                           (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(P, dS)");
     DSA_MARK(2);
-    bwd_dq_kernel<3><<<dim3(cnt), dim3(256), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start);
+    bwd_dq_kernel<3><<<dim3(cnt), dim3(512), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ)");
     DSA_MARK(3);
     bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, sids, pds, dstp, rows, q0, cnt,
