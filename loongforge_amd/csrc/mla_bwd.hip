@@ -307,7 +307,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
   for (int n = 0; n < ntiles; n++) {
     wait_vmcnt_le(per_issue * min(STAGES - 2, ntiles - 1 - n));
     __syncthreads();
-    if (n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
+    // The two waves of a SIMD (w, 0) and (w, 1) issue their transfers at different times - here and after
+    // the second d-tile - so that each does so while the other one feeds the matrix pipe.
+    if (hh == 0 && n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
     const unsigned char* tb = smem + (n % STAGES) * STAGE_BYTES;
     // the four dS operands of the wave's two head groups: [hg0 or hg1][k-step]
     bf16x8 bds[2][2];
@@ -344,6 +346,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+      if (i == 1) {
+        if (hh == 1 && n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
   // ---- write dQ: accumulator e of a lane is d = 32*dt + 8*(e/4) + 4*g + (e%4), head = 32*hg + r ----
