@@ -129,12 +129,10 @@ def main():
         e[0].record()
         # quantise q and k, fold the query scales into the head weights, logits + top-k: straight
         # through the C ABI on preallocated buffers, like the attention calls below
-        _lib.check(lib.dsa_quant_rowwise_e4m3(iq_d.data_ptr(), S * HI, 128, q8.data_ptr(), qs.data_ptr(), 1e-12, 1,
-                                              stream), "quant q")
+        _lib.check(lib.dsa_quant_rowwise_e4m3_weights(iq_d.data_ptr(), S * HI, 128, q8.data_ptr(), qs.data_ptr(), 1e-12, 1,
+                                                      0, w_d.data_ptr(), 128 ** -0.5, wsd.data_ptr(), stream), "quant q")
         _lib.check(lib.dsa_quant_rowwise_e4m3(ik_d.data_ptr(), S, 128, k8.data_ptr(), ksc.data_ptr(), 1e-12, 1,
                                               stream), "quant k")
-        torch.mul(w_d, qs, out=wsd)
-        wsd.mul_(128 ** -0.5)
         e[1].record()
         _lib.check(lib.dsa_indexer_topk_fwd(q8.data_ptr(), wsd.data_ptr(), k8.data_ptr(), ksc.data_ptr(), ks.data_ptr(),
                                             ke.data_ptr(), S, HI, S, K, 1, sc.data_ptr(), ids.data_ptr(),

@@ -53,6 +53,19 @@ int dsa_rotate_quant_e4m3(const void* x, int64_t rows, int cols, void* x8, float
                           float eps, int pow2, void* stream);
 
 /*
+ * The quantiser above (after the rotation when rotate != 0) that also writes, per row,
+ *   weight_scaled[row] = (weights[row] * scale_inv[row]) * factor
+ * i.e. the indexer's `weight_scaled = weights * q_scale * softmax_scale`
+ * (dsa_fused_kernels.py:2362, deepseek_v4_csa.py:1386) with rows = (token, head) and
+ * factor = head_dim^-0.5, in the same kernel that produces q_scale instead of two elementwise
+ * launches after it.  The products are rounded one after the other, as the separate operations are.
+ *   weights, weight_scaled [rows] f32
+ */
+int dsa_quant_rowwise_e4m3_weights(const void* x, int64_t rows, int cols, void* x8, float* scale_inv,
+                                   float eps, int pow2, int rotate, const float* weights, float factor,
+                                   float* weight_scaled, void* stream);
+
+/*
  * Lightning-indexer logits:
  *   logits[i, j - base_i] = k_scale[j] * sum_h q_w[i,h] * relu(q8[i,h,:] . k8[j,:]),  ks[i] <= j < ke[i]
  * and -inf for every other column of row i.  base_i = 0 when `relative` == 0 (dense layout, width

@@ -127,9 +127,8 @@ class CSAIndexerKernelFunction(torch.autograd.Function):
         q = _pad_to(index_q.squeeze(1).to(torch.bfloat16), head_p, 1).contiguous()
         k = index_k.squeeze(1).to(torch.bfloat16).contiguous()
         w = _pad_to(weights.squeeze(1).float(), head_p, 1)
-        q_fp8, q_scale = ops.quant_rowwise_e4m3(q)
+        q_fp8, q_scale, weight_scaled = ops.quant_rowwise_e4m3_weights(q, w, softmax_scale)
         k_fp8, k_scale = ops.quant_rowwise_e4m3(k)
-        weight_scaled = w * q_scale * softmax_scale
 
         row = torch.arange(sq, dtype=torch.int, device=device)
         if packed_seq_params is not None:

@@ -16,7 +16,8 @@ __device__ __forceinline__ float wave_max16(float v) {   // max over the 16 lane
 // cols == 128: 16 lanes per row, 4 rows per wave, 16 rows per 256-thread block.
 __global__ __launch_bounds__(256) void quant128_kernel(const uint4* __restrict__ x, uint2* __restrict__ x8,
                                                        float* __restrict__ scale_inv, int64_t rows,
-                                                       float eps, int pow2) {
+                                                       float eps, int pow2, const float* __restrict__ w_in,
+                                                       float w_factor, float* __restrict__ w_scaled) {
   int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   int sub = threadIdx.x & 15;
   bool live = row < rows;
@@ -45,7 +46,11 @@ __global__ __launch_bounds__(256) void quant128_kernel(const uint4* __restrict__
   hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], hi, true);
   if (live) {
     x8[row * 16 + sub] = make_uint2((unsigned)lo, (unsigned)hi);
-    if (sub == 0) scale_inv[row] = 1.0f / scale;
+    if (sub == 0) {
+      const float si = 1.0f / scale;
+      scale_inv[row] = si;
+      if (w_scaled) w_scaled[row] = (w_in[row] * si) * w_factor;      // two roundings, as two separate multiplications
+    }
   }
 }
 
@@ -56,7 +61,9 @@ __global__ __launch_bounds__(256) void quant128_kernel(const uint4* __restrict__
 // quantised payload only).
 __global__ __launch_bounds__(256) void rotate_quant128_kernel(const uint4* __restrict__ x, uint2* __restrict__ x8,
                                                               float* __restrict__ scale_inv, uint4* __restrict__ y,
-                                                              int64_t rows, float eps, int pow2) {
+                                                              int64_t rows, float eps, int pow2,
+                                                              const float* __restrict__ w_in, float w_factor,
+                                                              float* __restrict__ w_scaled) {
   int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   int sub = threadIdx.x & 15;
   bool live = row < rows;
@@ -107,7 +114,11 @@ __global__ __launch_bounds__(256) void rotate_quant128_kernel(const uint4* __res
   hi = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], hi, true);
   if (live) {
     x8[row * 16 + sub] = make_uint2((unsigned)lo, (unsigned)hi);
-    if (sub == 0) scale_inv[row] = 1.0f / scale;
+    if (sub == 0) {
+      const float si = 1.0f / scale;
+      scale_inv[row] = si;
+      if (w_scaled) w_scaled[row] = (w_in[row] * si) * w_factor;      // two roundings, as two separate multiplications
+    }
   }
 }
 
@@ -125,7 +136,7 @@ extern "C" int dsa_rotate_quant_e4m3(const void* x, int64_t rows, int cols, void
   int64_t blocks = (rows + 15) / 16;
   DSA_REQUIRE(blocks < (1ll << 31), "dsa_rotate_quant_e4m3: too many rows");
   rotate_quant128_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
-      (const uint4*)x, (uint2*)x8, scale_inv, (uint4*)y, rows, eps, pow2);
+      (const uint4*)x, (uint2*)x8, scale_inv, (uint4*)y, rows, eps, pow2, nullptr, 0.f, nullptr);
   DSA_CHECK_LAUNCH("dsa_rotate_quant_e4m3");
   return DSA_OK;
 }
@@ -139,7 +150,28 @@ extern "C" int dsa_quant_rowwise_e4m3(const void* x, int64_t rows, int cols, voi
   int64_t blocks = (rows + 15) / 16;
   DSA_REQUIRE(blocks < (1ll << 31), "dsa_quant_rowwise_e4m3: too many rows");
   quant128_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
-      (const uint4*)x, (uint2*)x8, scale_inv, rows, eps, pow2);
+      (const uint4*)x, (uint2*)x8, scale_inv, rows, eps, pow2, nullptr, 0.f, nullptr);
   DSA_CHECK_LAUNCH("dsa_quant_rowwise_e4m3");
+  return DSA_OK;
+}
+
+extern "C" int dsa_quant_rowwise_e4m3_weights(const void* x, int64_t rows, int cols, void* x8, float* scale_inv,
+                                              float eps, int pow2, int rotate, const float* weights, float factor,
+                                              float* weight_scaled, void* stream) {
+  DSA_REQUIRE(cols == 128, "dsa_quant_rowwise_e4m3_weights: only rows of 128 elements are supported, got %d", cols);
+  DSA_REQUIRE(rows >= 0, "dsa_quant_rowwise_e4m3_weights: negative row count");
+  DSA_REQUIRE(x8 != nullptr && scale_inv != nullptr && weights != nullptr && weight_scaled != nullptr,
+              "dsa_quant_rowwise_e4m3_weights: null pointer");
+  DSA_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)x8 % 8) == 0, "dsa_quant_rowwise_e4m3_weights: misaligned pointer");
+  if (rows == 0) return DSA_OK;
+  int64_t blocks = (rows + 15) / 16;
+  DSA_REQUIRE(blocks < (1ll << 31), "dsa_quant_rowwise_e4m3_weights: too many rows");
+  if (rotate)
+    rotate_quant128_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+        (const uint4*)x, (uint2*)x8, scale_inv, nullptr, rows, eps, pow2, weights, factor, weight_scaled);
+  else
+    quant128_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+        (const uint4*)x, (uint2*)x8, scale_inv, rows, eps, pow2, weights, factor, weight_scaled);
+  DSA_CHECK_LAUNCH("dsa_quant_rowwise_e4m3_weights");
   return DSA_OK;
 }

@@ -234,7 +234,9 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
         # quantiser (a zero-padded head dimension cannot be rotated after padding: 128 only)
         assert not rotate or dim == 128, "the fused rotation needs head dim 128"
         quant = ops.rotate_quant_e4m3 if rotate else ops.quant_rowwise_e4m3
-        q_fp8, q_scale = quant(q_p)
+        # weight_scaled = weights * q_scale * softmax_scale comes out of the query's quantiser kernel
+        q_fp8, q_scale, weight_scaled = ops.quant_rowwise_e4m3_weights(q_p, _pad_to(weights.float(), head_p, 1),
+                                                                       softmax_scale, rotate)
         k_fp8, k_scale = quant(k_p)
 
         if packed_seq_params is None:
@@ -250,7 +252,6 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
             k_start = cu[local_seq_ids.long()].int()
         k_end = torch.arange(seq_q, dtype=torch.int, device=device) + chunk_offset + 1
 
-        weight_scaled = _pad_to(weights.float(), head_p, 1) * q_scale * softmax_scale
         index_score_topk, topk_indices = ops.indexer_topk(q_fp8, weight_scaled, k_fp8, k_scale, k_start, k_end,
                                                           index_topk, DSAIndexerKernelFunction.sorted_output)
         ctx.softmax_scale = softmax_scale

@@ -99,6 +99,43 @@ def rotate_quant_e4m3(x: torch.Tensor, eps: float = 1e-12, pow2: bool = True, re
     return (x8.view(_FP8), scale_inv, y) if return_rotated else (x8.view(_FP8), scale_inv)
 
 
+@torch.library.custom_op("dsa::quant_rowwise_e4m3_weights", mutates_args=())
+def _quant_weights_op(x: torch.Tensor, weights: torch.Tensor, factor: float, rotate: bool, eps: float,
+                      pow2: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _need_gpu(x, weights)
+    if x.dtype != torch.bfloat16 or x.shape[-1] != 128:
+        raise ValueError("quant_rowwise_e4m3_weights expects bf16 rows of 128 elements")
+    if weights.shape != x.shape[:-1]:
+        raise ValueError("quant_rowwise_e4m3_weights: one weight per row expected, got %s for rows %s"
+                         % (tuple(weights.shape), tuple(x.shape[:-1])))
+    x, weights = _c(x), _c(weights.float())
+    rows = x.numel() // 128
+    x8 = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    scale_inv = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    w_scaled = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        _lib.check(lib.dsa_quant_rowwise_e4m3_weights(x.data_ptr(), rows, 128, x8.data_ptr(), scale_inv.data_ptr(),
+                                                      float(eps), int(pow2), int(rotate), weights.data_ptr(),
+                                                      float(factor), w_scaled.data_ptr(), _stream(x)),
+                   "dsa_quant_rowwise_e4m3_weights")
+    return x8, scale_inv, w_scaled
+
+
+@_quant_weights_op.register_fake
+def _(x, weights, factor, rotate, eps, pow2):
+    return (x.new_empty(x.shape, dtype=torch.uint8), x.new_empty(x.shape[:-1], dtype=torch.float32),
+            x.new_empty(x.shape[:-1], dtype=torch.float32))
+
+
+def quant_rowwise_e4m3_weights(x: torch.Tensor, weights: torch.Tensor, factor: float, rotate: bool = False,
+                               eps: float = 1e-12, pow2: bool = True):
+    """:func:`quant_rowwise_e4m3` (after the Hadamard rotation when ``rotate``) that also returns
+    ``(weights * scale_inv) * factor`` per row: (fp8 payload, ``scale_inv``, scaled weights fp32)."""
+    x8, scale_inv, w_scaled = _quant_weights_op(x, weights, float(factor), bool(rotate), eps, pow2)
+    return x8.view(_FP8), scale_inv, w_scaled
+
+
 def rotate_bf16(x: torch.Tensor):
     """Hadamard rotation of bf16 rows of 128 (x 128^-0.5), the kernel form of ``rotate_activation``."""
     return _rotate_quant_op(x, 1e-12, True, False, True)[2]

@@ -230,6 +230,22 @@ def test_fused_rotation_and_quantiser(gpu):
     assert (back - x.float()).abs().max().item() <= 2.0 ** -6 * x.float().abs().max().item()
 
 
+def test_quantiser_with_weight_scaling_equals_the_separate_operations(gpu):
+    """The quantiser kernel that also emits weights * scale_inv * factor: payload and scales are those
+    of the plain kernel, the scaled weights are bit-equal to the two torch multiplications."""
+    from loongforge_amd import ops
+
+    iq, _, w = O.make_indexer_inputs(300, 64, 128, seed=3)
+    x, wd = iq.to(gpu), w.to(gpu)
+    for rotate in (False, True):
+        plain = ops.rotate_quant_e4m3(x) if rotate else ops.quant_rowwise_e4m3(x)
+        x8, si, ws = ops.quant_rowwise_e4m3_weights(x, wd, 128 ** -0.5, rotate)
+        assert torch.equal(x8.view(torch.uint8), plain[0].view(torch.uint8)) and torch.equal(si, plain[1])
+        assert torch.equal(ws, wd * si * 128 ** -0.5)
+    with pytest.raises(ValueError):
+        ops.quant_rowwise_e4m3_weights(x, wd[:, :32], 1.0)
+
+
 def test_indexer_kernel_with_fused_rotation_matches_rotating_first(gpu):
     """DSAIndexerKernel(rotate=True) == DSAIndexerKernel on pre-rotated inputs: same scores and ids, and
     gradients that agree with autograd through rotate_activation."""
