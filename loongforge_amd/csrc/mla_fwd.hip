@@ -62,23 +62,17 @@ __device__ __forceinline__ void mfma_chain_done(f32x16& acc) {
 // true row maximum with an extra sweep of S^T over all tiles.
 constexpr unsigned LSE_REDO_MARK = 0x7fc0d5a0u;
 
+// One query, by the 256 threads of a workgroup.
 template <int STAGES, int POUT, bool EXACT>   // POUT: 0 none, 1 bf16, 2 f32
-__global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
+__device__ __forceinline__ void fwd_query(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
     __bf16* __restrict__ out, float* __restrict__ lse, void* __restrict__ p_out,
-    int S, int H, int Skv, int K, int q_start, float sm_scale, const float* __restrict__ sink, int p_skip) {
+    int S, int H, int Skv, int K, int q_start, float sm_scale, const float* __restrict__ sink, int p_skip, int qi) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, g = lane >> 5;
-  const int qi = S - 1 - (int)blockIdx.x;          // longest prefixes first
   const int qpos = q_start + qi;
   const int NT = K / BI;
-  if (EXACT) {   // only queries the fast pass marked
-    const unsigned* lw = (const unsigned*)lse + (size_t)qi * H;
-    bool redo = false;
-    for (int w = 0; w * 32 < H; w++) redo |= (lw[w * 32] == LSE_REDO_MARK);
-    if (!redo) return;
-  }
 
   int* idx_s = (int*)(smem + STAGES * TILE_BYTES);
   unsigned* tmask = (unsigned*)(idx_s + K);
@@ -363,6 +357,36 @@ __global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
   }
 }
 
+// Fast pass: workgroup b takes query S - 1 - b (longest prefixes first).  Exact pass: workgroup b
+// looks at the marks of queries 32b .. 32b + 31 with one load per lane and redoes the marked ones,
+// so that a launch in which nothing is marked costs a few microseconds, not a full-size workgroup
+// per query.
+template <int STAGES, int POUT, bool EXACT>
+__global__ __launch_bounds__(256, 1) void mla_fwd_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
+    __bf16* __restrict__ out, float* __restrict__ lse, void* __restrict__ p_out,
+    int S, int H, int Skv, int K, int q_start, float sm_scale, const float* __restrict__ sink, int p_skip) {
+  if (!EXACT) {
+    fwd_query<STAGES, POUT, false>(q, kv, ids, out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip,
+                                   S - 1 - (int)blockIdx.x);
+    return;
+  }
+  const int qc = (int)blockIdx.x * 32 + (int)(threadIdx.x & 31);
+  bool redo = false;
+  if (qc < S) {
+    const unsigned* lw = (const unsigned*)lse + (size_t)qc * H;
+    for (int w = 0; w * 32 < H; w++) redo |= (lw[w * 32] == LSE_REDO_MARK);
+  }
+  unsigned todo = (unsigned)__ballot(redo);      // every wave reads the same 32 marks before any of them is rewritten
+  while (todo) {
+    const int b = __builtin_ctz(todo);
+    todo &= todo - 1;
+    fwd_query<STAGES, POUT, true>(q, kv, ids, out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip,
+                                  (int)blockIdx.x * 32 + b);
+    __syncthreads();
+  }
+}
+
 template <int STAGES>
 int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, int Skv, int K, int q_start,
                float sm_scale, void* out, float* lse, void* p_out, int p_out_f32, const float* sink, int p_skip, hipStream_t st) {
@@ -375,7 +399,7 @@ int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, 
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2; \
     if (hipFuncSetAttribute((const void*)kern2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2; \
     kern<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip); \
-    kern2<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip); \
+    kern2<<<dim3((S + 31) / 32), block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip); \
   } while (0)
   if (!p_out) DSA_FWD_LAUNCH(0);
   else if (!p_out_f32) DSA_FWD_LAUNCH(1);
