@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
   float* stat_s = (float*)(ntile_s + 4);       // [2][128]: lse * log2(e), delta
-  const int ntiles = stage_ids(ids, qi, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
+  const int ntiles = stage_ids(ids, ql, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
 
   const int h = wave * 32 + r;
   const bool head_ok = h < H;
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
   // (the helper is written for four waves; the other four repeat part of its work with equal results)
-  const int ntiles = stage_ids(ids, qi, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
+  const int ntiles = stage_ids(ids, ql, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
 
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
   const LaneOffsets lo = lane_offsets();
@@ -417,7 +417,7 @@ __device__ __forceinline__ void dkv_body(
     for (int i = 0; i < 8; i++)       // invalid slots land in a scratch row: the store count stays fixed
       if (t0 + i * 256 < K + BI) dst_s[t0 + i * 256] = d[i] >= 0 ? d[i] : dummy_row;
   }
-  const int ntiles = stage_ids(ids, qi, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
+  const int ntiles = stage_ids(ids, ql, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
   if (ntiles == 0) return;
 
   // ---- X^T operands: x?[c][kk], kk = 2*w' + s' over the 8 groups of 16 heads ------------------
@@ -744,7 +744,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     // gather neighbouring latent rows at the same time.
     order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st, sorted);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
-    const int* sids = sorted - (size_t)q0 * K;          // indexed by global query, like ids
+    const int* sids = sorted;                           // row ql of the list belongs to query q0 + ql
     DSA_MARK(1);
     bwd_pds_kernel<4><<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out,
                                                           (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);

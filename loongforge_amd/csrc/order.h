@@ -135,14 +135,14 @@ static __global__ __launch_bounds__(1024) void key_scan_kernel(const int* __rest
 }
 
 // dst[ql][slot] = row of the pair in key-sorted order (-1 for invalid slots)
-static __global__ void rank_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv, int q_start,
+static __global__ void rank_kernel(const int* __restrict__ ids, int row0, int q0, int cnt, int K, int Skv, int q_start,
                             const unsigned* __restrict__ bitmap, const unsigned* __restrict__ prefix,
                             const int* __restrict__ start, int W, int* __restrict__ dst) {
   // blockIdx.y walks the queries, blockIdx.x the slots of one query in steps of the block size
   for (int ql = blockIdx.y; ql < cnt; ql += gridDim.y) {
     const int slot = blockIdx.x * blockDim.x + threadIdx.x;
     if (slot >= K) continue;
-    const int v = ids[(size_t)(q0 + ql) * K + slot];
+    const int v = ids[(size_t)(row0 + ql) * K + slot];      // row0: row of local query 0 in the id array handed in
     int d = -1;
     if (v >= 0 && v < Skv && v <= q_start + q0 + ql) {
       const size_t wi = (size_t)v * W + (ql >> 5);
@@ -178,9 +178,8 @@ inline void build(const int* ids, int q0, int cnt, int K, int Skv, int q_start, 
   bm_prefix_kernel<<<dim3((Skv + 3) / 4), dim3(256), 0, st>>>(bitmap, prefix, count, Skv, W);
   key_scan_kernel<<<dim3(1), dim3(1024), 0, st>>>(count, start, Skv);
   // with `sorted` (rows of the block's queries, [cnt][K]) the ranks are those of the sorted slots
-  const int* rank_ids = sorted ? sorted - (size_t)q0 * K : ids;
-  rank_kernel<<<dim3((K + 255) / 256, cnt < 32768 ? cnt : 32768), dim3(256), 0, st>>>(rank_ids, q0, cnt, K, Skv, q_start, bitmap,
-                                                                                     prefix, start, W, dst);
+  rank_kernel<<<dim3((K + 255) / 256, cnt < 32768 ? cnt : 32768), dim3(256), 0, st>>>(sorted ? sorted : ids, sorted ? 0 : q0, q0, cnt,
+                                                                                     K, Skv, q_start, bitmap, prefix, start, W, dst);
 }
 
 }  // namespace order
