@@ -151,8 +151,10 @@ class CSAIndexerKernelFunction(torch.autograd.Function):
             k_end = torch.div(row + (sq_offset + 1), compress_ratio, rounding_mode="floor").clamp(min=1, max=sk)
             effective_topk = min(index_topk, sk)
 
+        # the reference asks for unsorted output, i.e. any slot order will do: the descending-score path of the
+        # top-k kernel is its fast one
         index_score_topk, global_ids = ops.indexer_topk(q_fp8, weight_scaled, k_fp8, k_scale, k_start.int(),
-                                                        k_end.int(), effective_topk, False)
+                                                        k_end.int(), effective_topk, True)
         if packed_seq_params is not None:
             topk_indices = torch.where(global_ids >= 0, global_ids - k_start.unsqueeze(1), global_ids)
         else:
