@@ -3,6 +3,9 @@
 // w, w+4, ...; a head's K logits live in registers, so p_out is read exactly once.  Two variants:
 // 16-byte loads when the layout allows it, element loads otherwise (the same arithmetic; the partial
 // sums of a head are grouped differently, so results agree to fp32 rounding, not bit for bit).
+// exp2 is the bare hardware instruction (the arguments are <= 0; results below 2^-126 flush to zero):
+// the library routine's range handling costs four more instructions per logit, and this kernel is
+// bound by them.
 #include "dsa_common.h"
 
 namespace {
@@ -50,7 +53,7 @@ __global__ __launch_bounds__(256) void attn_dist_kernel(const void* __restrict__
     if (mx == -INFINITY) continue;            // head with no valid slot contributes nothing
     float sum = 0.f;
 #pragma unroll
-    for (int v = 0; v < NV; v++) { z[v] = exp2f(z[v] - mx); sum += z[v]; }
+    for (int v = 0; v < NV; v++) { z[v] = __builtin_amdgcn_exp2f(z[v] - mx); sum += z[v]; }
     sum = wave_sum(sum);
     float inv = 1.0f / sum;
 #pragma unroll
@@ -65,7 +68,8 @@ __global__ __launch_bounds__(256) void attn_dist_kernel(const void* __restrict__
 }
 
 // The same with 16-byte loads: lane l of a wave owns slots 8 (64 v + l) .. +7 of every head.  Needs
-// K, the strides and the base address to be multiples of 8 elements.
+// K, the strides and the base address to be multiples of 8 elements, and a positive scale (the row
+// maximum is taken on the raw logits).
 template <bool F32, int NC>
 __global__ __launch_bounds__(256) void attn_dist_vec_kernel(const void* __restrict__ p_out, int H, int K,
                                                             int64_t ld_s, int64_t ld_h, float c2,
@@ -108,13 +112,13 @@ __global__ __launch_bounds__(256) void attn_dist_vec_kernel(const void* __restri
         if (F32) {
           const unsigned w[8] = {cur.a[v].x, cur.a[v].y, cur.a[v].z, cur.a[v].w, cur.b[v].x, cur.b[v].y, cur.b[v].z, cur.b[v].w};
 #pragma unroll
-          for (int e = 0; e < 8; e++) z[v][e] = __builtin_bit_cast(float, w[e]) * c2;
+          for (int e = 0; e < 8; e++) z[v][e] = __builtin_bit_cast(float, w[e]);
         } else {
           const unsigned w[4] = {cur.a[v].x, cur.a[v].y, cur.a[v].z, cur.a[v].w};
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            z[v][2 * e] = __builtin_bit_cast(float, w[e] << 16) * c2;
-            z[v][2 * e + 1] = __builtin_bit_cast(float, w[e] & 0xffff0000u) * c2;
+            z[v][2 * e] = __builtin_bit_cast(float, w[e] << 16);
+            z[v][2 * e + 1] = __builtin_bit_cast(float, w[e] & 0xffff0000u);
           }
         }
       } else {
@@ -127,11 +131,13 @@ __global__ __launch_bounds__(256) void attn_dist_vec_kernel(const void* __restri
     cur = nxt;
     mx = wave_max(mx);
     if (mx == -INFINITY) continue;            // head with no valid slot contributes nothing
+    // the (positive) scale enters through one fused multiply-add per logit: exp2(z c2 - max(z) c2)
+    const float off = -mx * c2;
     float sum = 0.f;
 #pragma unroll
     for (int v = 0; v < NC; v++)
 #pragma unroll
-      for (int e = 0; e < 8; e++) { z[v][e] = exp2f(z[v][e] - mx); sum += z[v][e]; }
+      for (int e = 0; e < 8; e++) { z[v][e] = __builtin_amdgcn_exp2f(fmaf(z[v][e], c2, off)); sum += z[v][e]; }
     sum = wave_sum(sum);
     const float inv = 1.0f / sum;
 #pragma unroll
@@ -158,7 +164,7 @@ int launch(const void* p_out, int S, int H, int K, int64_t ld_s, int64_t ld_h, f
            hipStream_t st) {
   const float c2 = sm_scale * 1.4426950408889634f;
   size_t smem = (size_t)4 * K * sizeof(float);
-  const bool vec = K % 8 == 0 && ld_s % 8 == 0 && ld_h % 8 == 0 && ((uintptr_t)p_out % 32) == 0;
+  const bool vec = K % 8 == 0 && ld_s % 8 == 0 && ld_h % 8 == 0 && ((uintptr_t)p_out % 32) == 0 && c2 > 0.f;
   if (vec) {
     const int nc = (K + 511) / 512;
 #define DSA_ADV_CASE(N) \
