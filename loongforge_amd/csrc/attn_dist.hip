@@ -99,10 +99,8 @@ __global__ __launch_bounds__(256) void attn_dist_vec_kernel(const void* __restri
       }
     }
   };
-  Raw cur, nxt;
-  fetch(wave, cur);
-  for (int h = wave; h < H; h += 4) {
-    fetch(h + 4, nxt);
+  // one head: its softmax numerators, their sum, and the accumulation of the normalised values
+  auto head = [&](const Raw& cur) {
     float z[NC][8];
     float mx = -INFINITY;
 #pragma unroll
@@ -128,9 +126,8 @@ __global__ __launch_bounds__(256) void attn_dist_vec_kernel(const void* __restri
 #pragma unroll
       for (int e = 0; e < 8; e++) mx = fmaxf(mx, z[v][e]);
     }
-    cur = nxt;
     mx = wave_max(mx);
-    if (mx == -INFINITY) continue;            // head with no valid slot contributes nothing
+    if (mx == -INFINITY) return;              // head with no valid slot contributes nothing
     // the (positive) scale enters through one fused multiply-add per logit: exp2(z c2 - max(z) c2)
     const float off = -mx * c2;
     float sum = 0.f;
@@ -144,6 +141,17 @@ __global__ __launch_bounds__(256) void attn_dist_vec_kernel(const void* __restri
     for (int v = 0; v < NC; v++)
 #pragma unroll
       for (int e = 0; e < 8; e++) acc[v][e] += z[v][e] * inv;
+  };
+  // two buffers take turns (no register copies): while one head is worked on, the next is on its way
+  Raw r0, r1;
+  fetch(wave, r0);
+  for (int h = wave; h < H; h += 8) {
+    fetch(h + 4, r1);
+    head(r0);
+    if (h + 4 < H) {
+      fetch(h + 8, r0);
+      head(r1);
+    }
   }
 #pragma unroll
   for (int v = 0; v < NC; v++) {
