@@ -235,6 +235,13 @@ def main():
                  "stream_read_gbps": round(row_bytes / (t_read * 1e-3) / 1e9, 1),
                  "note": "plain movers with the byte counts and access shape of bwd_dkv_kernel and bwd_reduce_kernel"}
 
+    # what the matrix pipes sustain when a kernel issues nothing but bf16 MFMAs (about 20 ms of them)
+    probe_flops = ctypes.c_double(0.0)
+    sink4 = torch.zeros(4, dtype=torch.float32, device=dev)
+    t_mfma, _ = timed(lambda: _lib.check(lib.dsa_probe_mfma_bf16(2048, 10000, sink4.data_ptr(), ctypes.byref(probe_flops),
+                                                                 stream), "probe mfma"))
+    mfma_sustained = probe_flops.value / (t_mfma * 1e-3) / 1e12
+
     mla_tflops = (flops_fwd + flops_bwd) / ((t_fwd + t_bwd) * 1e-3) / 1e12
     # ---- roofline of the longest-running kernel of the step ---------------------------------------
     # Per kernel: algorithmic flops and algorithmic HBM bytes of one launch.  Gathered key rows are
@@ -316,6 +323,8 @@ def main():
         "rope_permute_cat_ms": round(t_rope, 3),
         "rope_permute_cat_gbps": round(4.0 * S * H * DQK / (t_rope * 1e-3) / 1e9, 1),
         "wall_s_per_step": round(wall / n, 4),
+        "mfma_bf16_sustained_tflops": round(mfma_sustained, 1),
+        "frac_of_sustained_bf16_mfma": round(mla_tflops / mfma_sustained, 4),
         "hbm_plain_mover": mover,
         "roofline": roofline,
     }

@@ -234,8 +234,9 @@ int dsa_rope_headsum_inverse(const void* grad, int64_t g_tok, int64_t g_head, vo
 
 /*
  * Measurement aids; no counterpart in the reference.  Plain data movers with the traffic shape of
- * the two bandwidth-bound backward passes, so that a benchmark can quote those passes against what
- * the memory system gives a kernel that does nothing else.
+ * the two bandwidth-bound backward passes, and a kernel of nothing but bf16 MFMAs, so that a
+ * benchmark can quote the kernels against what the memory system and the matrix pipes give a
+ * kernel that does nothing else.
  *
  * dsa_probe_hbm_rows: `workgroups` x `rows_per_workgroup` (a multiple of 4) rows of 1152 bytes are
  * written to `rows` (at permuted row positions when scatter != 0, in order otherwise) while each
@@ -247,6 +248,9 @@ int dsa_rope_headsum_inverse(const void* grad, int64_t g_tok, int64_t g_head, vo
 int dsa_probe_hbm_rows(const void* src, void* rows, int workgroups, int rows_per_workgroup, int read_fifths,
                        int scatter, void* stream);
 int dsa_probe_hbm_read(const void* src, size_t bytes, void* sink16, void* stream);
+/* dsa_probe_mfma_bf16: `workgroups` x 4 waves each issue iters x 16 v_mfma_f32_32x32x16_bf16 and nothing else;
+ * *flops (may be NULL) receives the flop count of the launch; sink4 points at 4 writable bytes. */
+int dsa_probe_mfma_bf16(int workgroups, int iters, void* sink4, double* flops, void* stream);
 
 #ifdef __cplusplus
 }

@@ -37,6 +37,7 @@ SIGNATURES = {
     "dsa_rope_headsum_inverse": (_i, [_vp, _i64, _i64, _vp, _i64, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
     "dsa_probe_hbm_rows": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "dsa_probe_hbm_read": (_i, [_vp, _sz, _vp, _vp]),
+    "dsa_probe_mfma_bf16": (_i, [_i, _i, _vp, _vp, _vp]),
 }
 
 _lib = None

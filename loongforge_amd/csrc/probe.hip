@@ -45,7 +45,47 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = acc;     // keeps the loads alive; practically never taken
 }
 
+// Nothing but bf16 MFMAs: each wave runs `iters` rounds of 16 back-to-back v_mfma_f32_32x32x16_bf16 on four
+// independent accumulators with non-trivial operands; what the matrix pipes sustain at the clock the
+// part holds under that load.
+__global__ __launch_bounds__(256, 1) void probe_mfma_kernel(float* __restrict__ sink, int iters) {
+  const int lane = threadIdx.x & 63;
+  bf16x8 a, b;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    // pseudo-random values in [-1, 1): operands with busy mantissa bits (the clock the part holds depends
+    // on how many bits toggle; all-zero operands run a fifth faster)
+    const unsigned ha = (unsigned)(lane * 8 + e + 1) * 2654435761u, hb = (unsigned)(lane * 8 + e + 977) * 2246822519u;
+    a[e] = (__bf16)((float)(ha >> 16) * (1.0f / 32768.0f) - 1.0f);
+    b[e] = (__bf16)((float)(hb >> 16) * (1.0f / 32768.0f) - 1.0f);
+  }
+  f32x16 acc[4];
+#pragma unroll
+  for (int u = 0; u < 4; u++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[u][e] = 0.f;
+  for (int it = 0; it < iters; it++) {
+    asm volatile("" : "+v"(a), "+v"(b));          // keeps the loop body in the loop
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+      for (int u = 0; u < 4; u++) acc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[u], 0, 0, 0);
+  }
+  float keep = 0.f;
+#pragma unroll
+  for (int u = 0; u < 4; u++) keep += acc[u][0];
+  if (keep == 123.456f) sink[0] = keep;           // practically never taken
+}
+
 }  // namespace
+
+extern "C" int dsa_probe_mfma_bf16(int workgroups, int iters, void* sink4, double* flops, void* stream) {
+  DSA_REQUIRE(workgroups > 0 && iters > 0 && sink4 != nullptr, "dsa_probe_mfma_bf16: bad arguments");
+  probe_mfma_kernel<<<dim3(workgroups), dim3(256), 0, (hipStream_t)stream>>>((float*)sink4, iters);
+  DSA_CHECK_LAUNCH("dsa_probe_mfma_bf16");
+  if (flops) *flops = (double)workgroups * 4.0 * (double)iters * 16.0 * (2.0 * 32 * 32 * 16);
+  return DSA_OK;
+}
 
 extern "C" int dsa_probe_hbm_rows(const void* src, void* rows, int workgroups, int rows_per_workgroup, int read_fifths,
                                   int scatter, void* stream) {
