@@ -742,9 +742,12 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     // The passes are free to choose their slot order (P, dS and the dKV rows never leave the workspace):
     // they walk each query's valid ids in ascending key order, so that the queries in flight on an XCD
     // gather neighbouring latent rows at the same time.
-    order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st, sorted);
+    // (The list is put together in LDS next to a bitmap over all keys; with more keys than fit there the
+    // passes walk the caller's slot order instead.)
+    const bool sort_ids = order::sorted_list_fits(Skv, K);
+    order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st, sort_ids ? sorted : nullptr);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
-    const int* sids = sorted;                           // row ql of the list belongs to query q0 + ql
+    const int* sids = sort_ids ? sorted : ids + (size_t)q0 * K;      // row ql belongs to query q0 + ql
     DSA_MARK(1);
     bwd_pds_kernel<4><<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out,
                                                           (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);

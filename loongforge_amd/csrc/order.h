@@ -165,6 +165,10 @@ inline size_t prefix_words(int chunk, int Skv) {
   const size_t W = (size_t)(chunk + 31) / 32, Wk = (size_t)(Skv + 31) / 32;
   return (size_t)Skv * W > (size_t)chunk * Wk ? (size_t)Skv * W : (size_t)chunk * Wk;
 }
+// LDS of the first kernel with the sorted list: bitmap and prefix counts over all keys plus the list
+inline bool sorted_list_fits(int Skv, int K) {
+  return (size_t)((Skv + 31) / 32) * 8 + (size_t)K * 4 <= (size_t)150 * 1024;
+}
 inline void build(const int* ids, int q0, int cnt, int K, int Skv, int q_start, unsigned* bitmap, unsigned* prefix,
                   int* count, int* start, int* dst, int W, hipStream_t st, int* sorted = nullptr) {
   const int Wk = (Skv + 31) / 32;

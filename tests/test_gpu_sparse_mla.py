@@ -150,6 +150,37 @@ def test_backward_does_not_depend_on_the_slot_order(gpu):
     assert_close(dkv2, rdkv, "dkv", scale_aware=True)
 
 
+def test_backward_with_more_keys_than_the_key_bitmap_in_lds_holds(gpu):
+    """Beyond about 600 000 keys the per-query key bitmap (and with it the key-sorted id list) no longer
+    fits LDS and the passes walk the caller's slot order; results must not care.  The oracle runs on the
+    selected keys only (compacted), everything else must get a zero gradient."""
+    from loongforge_amd import ops
+
+    S, H, K, skv = 64, 128, 64, 620_000
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn(S, H, 576, generator=g).to(torch.bfloat16)
+    dout = torch.randn(S, H, 512, generator=g).to(torch.bfloat16)
+    picked = torch.randperm(skv, generator=g)[:1500]                       # the keys any query may select
+    kv_small = torch.randn(1500, 576, generator=g).to(torch.bfloat16)
+    idx_small = torch.stack([torch.randperm(1500, generator=g)[:K] for _ in range(S)]).to(torch.int32)
+    idx_small[3, 10:] = -1
+    idx = torch.where(idx_small >= 0, picked[idx_small.clamp(min=0).long()].to(torch.int32), idx_small)
+    kv = torch.zeros(skv, 576, dtype=torch.bfloat16)
+    kv[picked] = kv_small
+    sm = 192 ** -0.5
+    qd, kd, dd, ids = q.to(gpu), kv.to(gpu), dout.to(gpu), idx.to(gpu)
+    out, lse, _ = ops.sparse_mla_fwd(qd, kd, ids, skv, sm)                 # q_start = skv: no causal test
+    dq, dkv = ops.sparse_mla_bwd(qd, kd, out, dd, ids, lse, skv, sm)
+    ro, _, _ = O.sparse_mla_fwd(q, kv_small, idx_small, 1500, sm, 512)
+    rdq, rdkv = O.sparse_mla_bwd(q, kv_small, idx_small, dout, 1500, sm, 512)
+    assert_close(out, ro, "out")
+    assert_close(dq, rdq, "dq", scale_aware=True)
+    assert_close(dkv[picked.to(gpu)], rdkv, "dkv of the selected keys", scale_aware=True)
+    rest = torch.ones(skv, dtype=torch.bool)
+    rest[picked] = False
+    assert (dkv.cpu()[rest] == 0).all()
+
+
 def test_forward_and_backward_with_attention_sink(gpu):
     from loongforge_amd import ops
 
