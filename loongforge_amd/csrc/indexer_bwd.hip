@@ -444,6 +444,7 @@ extern "C" int dsa_indexer_bwd(const float* g, const void* q8, const void* k8, c
   DSA_REQUIRE(S >= 0 && Sk > 0, "dsa_indexer_bwd: bad sizes S=%d Sk=%d", S, Sk);
   DSA_REQUIRE(K > 0 && K % TK == 0 && K <= 4096, "dsa_indexer_bwd: top-k must be a multiple of 128 up to 4096, got %d", K);
   DSA_REQUIRE((size_t)Sk * D <= 0xffffffffull, "dsa_indexer_bwd: key array too large");
+  DSA_REQUIRE(Sk <= order::MAX_KEYS, "dsa_indexer_bwd: at most %d keys are supported, got %d", order::MAX_KEYS, Sk);
   DSA_REQUIRE(((uintptr_t)q8 % 16) == 0 && ((uintptr_t)k8 % 16) == 0 && ((uintptr_t)q_w % 16) == 0 &&
               ((uintptr_t)d_q8 % 16) == 0 && ((uintptr_t)d_k8 % 16) == 0 && ((uintptr_t)workspace % 256) == 0,
               "dsa_indexer_bwd: misaligned pointer");

@@ -699,6 +699,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   DSA_REQUIRE(H > 0 && H <= 128 && H % 32 == 0, "dsa_sparse_mla_bwd: head count must be 32, 64, 96 or 128, got %d", H);
   DSA_REQUIRE(K > 0 && K % 64 == 0 && K <= 2048, "dsa_sparse_mla_bwd: top-k must be a multiple of 64 up to 2048, got %d", K);
   DSA_REQUIRE((size_t)Skv * DQK * 2 <= 0xffffffffull, "dsa_sparse_mla_bwd: kv larger than 4 GiB is not supported");
+  DSA_REQUIRE(Skv <= order::MAX_KEYS, "dsa_sparse_mla_bwd: at most %d keys are supported, got %d", order::MAX_KEYS, Skv);
   DSA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)kv % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
               ((uintptr_t)dout % 16) == 0 && ((uintptr_t)dq % 16) == 0 && ((uintptr_t)workspace % 256) == 0,
               "dsa_sparse_mla_bwd: misaligned pointer");

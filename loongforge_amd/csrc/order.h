@@ -165,6 +165,8 @@ inline size_t prefix_words(int chunk, int Skv) {
   const size_t W = (size_t)(chunk + 31) / 32, Wk = (size_t)(Skv + 31) / 32;
   return (size_t)Skv * W > (size_t)chunk * Wk ? (size_t)Skv * W : (size_t)chunk * Wk;
 }
+// The first kernel keeps one bit per key in LDS: the largest key count the builder takes
+constexpr int MAX_KEYS = 150 * 1024 * 8;
 // LDS of the first kernel with the sorted list: bitmap and prefix counts over all keys plus the list
 inline bool sorted_list_fits(int Skv, int K) {
   return (size_t)((Skv + 31) / 32) * 8 + (size_t)K * 4 <= (size_t)150 * 1024;

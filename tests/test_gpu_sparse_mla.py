@@ -267,3 +267,9 @@ def test_argument_errors(gpu):
         ops.sparse_mla_fwd(q[:, :16].contiguous(), kv, torch.zeros(8, 64, dtype=torch.int32, device=gpu))
     with pytest.raises(ValueError, match="d_v"):
         ops.sparse_mla_fwd(q, kv, torch.zeros(8, 64, dtype=torch.int32, device=gpu), d_v=256)
+    # the backward keeps one bit per key in LDS: more than 1 228 800 keys are turned down with a message
+    big = torch.zeros(1_300_000, 576, dtype=torch.bfloat16, device=gpu)
+    ids = torch.zeros(8, 64, dtype=torch.int32, device=gpu)
+    out, lse, _ = ops.sparse_mla_fwd(q, big, ids, 1_300_000)
+    with pytest.raises(ValueError, match="at most"):
+        ops.sparse_mla_bwd(q, big, out, torch.zeros_like(out), ids, lse, 1_300_000)
