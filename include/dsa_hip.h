@@ -110,7 +110,8 @@ int dsa_indexer_topk_fwd(const void* q8, const float* q_w, const void* k8, const
  *   d_qw[i,h]   = sum_t g[i,t] k_scale[j] relu(r_h)
  *   d_q8[i,h,:] = sum_t g[i,t] k_scale[j] q_w[i,h] [r_h > 0] k8[j,:]
  *   d_k8[j,:]   = sum_{(i,t): ids[i,t]=j} g[i,t] k_scale[j] sum_h q_w[i,h] [r_h > 0] q8[i,h,:]
- * d_k8 is accumulated in a fixed order (bit-reproducible).  Replaces
+ * d_k8 is accumulated in a fixed order (bit-reproducible); the ids of one query must be distinct
+ * (a row with a repeated id makes the call return d_k8 filled with NaN).  Replaces
  * lightning_indexer_bwd.fp8_mqa_logits_bwd as called at dsa_fused_kernels.py:2421-2430.
  *   g [S, K] f32   d_q8 [S, Hi, 128] f32   d_k8 [Sk, 128] f32   d_qw [S, Hi] f32
  */
@@ -155,8 +156,12 @@ int dsa_sparse_mla_fwd_ex(const void* q, const void* kv, const int32_t* ids, int
 
 /*
  * Sparse MQA-MLA attention backward: dQ and dKV of dsa_sparse_mla_fwd given dO, the saved out and
- * natural-log lse.  dKV is accumulated in fp32 in a fixed order (bit-reproducible, no float
- * atomics) and returned as bf16.  Replaces flash_mla_bwd.flash_mla_sparse_bwd /
+ * natural-log lse.  P and dS enter the matrix products as bf16 (as in the reference's kernel); the
+ * contribution of one (query, key) pair to dKV - a row of 576 values, summed over all heads in
+ * fp32 - is rounded to bf16 once, and the rows of a key are then summed in fp32 in a fixed order
+ * (bit-reproducible, no float atomics); dKV is returned as bf16.  The ids of one query must be
+ * distinct (any top-k is): a row with a repeated valid id makes the call return dq and dkv filled
+ * with NaN rather than sums that miss a term.  Replaces flash_mla_bwd.flash_mla_sparse_bwd /
  * sparse_mla_bwd_interface as called at dsa_fused_kernels.py:2086-2110
  * (math: loongforge/models/common/experimental_attention_variant/sparse_mla_bwd.py:292-356).
  *   dout [S, H, 512] bf16   dq [S, H, 576] bf16   dkv [Skv, 576] bf16

@@ -371,7 +371,8 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
 // d_k8[key] (+)= sum of the key's bf16 rows in fp32, ascending query order; 128 threads = 16 chunks of 8
 // columns x 8 row groups (row r of the segment goes to group r % 8), the groups combined in a fixed order
 __global__ __launch_bounds__(128) void indexer_reduce_kernel(const unsigned short* __restrict__ rows, const int* __restrict__ start,
-                                                             float* __restrict__ d_k8, int accumulate) {
+                                                             float* __restrict__ d_k8, int accumulate,
+                                                             const int* __restrict__ dup_flag) {
   __shared__ float part[8][D];
   const int key = blockIdx.x, ch = threadIdx.x & 15, grp = threadIdx.x >> 4;
   const int s0 = start[key], s1 = start[key + 1];
@@ -395,13 +396,14 @@ __global__ __launch_bounds__(128) void indexer_reduce_kernel(const unsigned shor
     float s = ((part[0][c] + part[1][c]) + (part[2][c] + part[3][c])) + ((part[4][c] + part[5][c]) + (part[6][c] + part[7][c]));
     float* p = d_k8 + (size_t)key * D + c;
     if (accumulate) s += *p;
+    if (*dup_flag) s = __builtin_nanf("");       // a query row held a repeated id: no sum that misses a term
     *p = s;
   }
 }
 
 struct Plan {
   int chunk, W;
-  size_t off_bitmap, off_prefix, off_count, off_start, off_dst, off_rows, total;
+  size_t off_bitmap, off_prefix, off_count, off_start, off_flag, off_dst, off_rows, total;
 };
 size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 Plan layout_plan(int chunk, int Sk, int K) {
@@ -413,6 +415,7 @@ Plan layout_plan(int chunk, int Sk, int K) {
   p.off_prefix = o; o = align_up(o + order::prefix_words(chunk, Sk) * 4);
   p.off_count = o; o = align_up(o + (size_t)(Sk + 1) * 4);
   p.off_start = o; o = align_up(o + (size_t)(Sk + 1) * 4);
+  p.off_flag = o; o = align_up(o + 4);
   p.off_dst = o; o = align_up(o + (size_t)chunk * K * 4);
   p.off_rows = o; o = align_up(o + ((size_t)chunk * K + 1) * D * 2);
   p.total = o;
@@ -458,6 +461,7 @@ extern "C" int dsa_indexer_bwd(const float* g, const void* q8, const void* k8, c
   unsigned* prefix = (unsigned*)(ws + p.off_prefix);
   int* count = (int*)(ws + p.off_count);
   int* start = (int*)(ws + p.off_start);
+  int* dup_flag = (int*)(ws + p.off_flag);
   int* dstp = (int*)(ws + p.off_dst);
   unsigned short* rows = (unsigned short*)(ws + p.off_rows);
   size_t smem = (size_t)2 * TILE_BYTES + 4 * 32 * 256 + 4 * 2 * 32 * 128 + (size_t)K * 12 + 4 * 64 * 4 + 4 * 32 * STRIP_STRIDE;
@@ -467,15 +471,16 @@ extern "C" int dsa_indexer_bwd(const float* g, const void* q8, const void* k8, c
   if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
     DSA_FAIL(DSA_ERR_LAUNCH, "dsa_indexer_bwd: cannot reserve LDS");
   bool first = true;
+  order::clear_flag(dup_flag, st);
   for (int q0 = 0; q0 < S; q0 += p.chunk) {
     const int cnt = S - q0 < p.chunk ? S - q0 : p.chunk;
     // every id inside [0, Sk) counts: the causal window was already applied when the ids were selected
-    order::build(ids, q0, cnt, K, Sk, 0x3fffffff, bitmap, prefix, count, start, dstp, p.W, st);
+    order::build(ids, q0, cnt, K, Sk, 0x3fffffff, bitmap, prefix, count, start, dstp, p.W, st, dup_flag);
     DSA_CHECK_LAUNCH("dsa_indexer_bwd(order)");
     kern<<<dim3(cnt), dim3(256), smem, st>>>(g, (const unsigned char*)q8, (const unsigned char*)k8, k_scale, q_w, ids, dstp,
                                              rows, d_q8, d_qw, q0, cnt, Sk, K, p.chunk * K);
     DSA_CHECK_LAUNCH("dsa_indexer_bwd");
-    indexer_reduce_kernel<<<dim3(Sk), dim3(128), 0, st>>>(rows, start, d_k8, first ? 0 : 1);
+    indexer_reduce_kernel<<<dim3(Sk), dim3(128), 0, st>>>(rows, start, d_k8, first ? 0 : 1, dup_flag);
     DSA_CHECK_LAUNCH("dsa_indexer_bwd(reduce)");
     first = false;
   }

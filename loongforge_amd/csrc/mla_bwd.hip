@@ -211,7 +211,7 @@ __global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
 template <int STAGES>
 __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
     const __bf16* __restrict__ kv, const int* __restrict__ ids, const unsigned char* __restrict__ pds,
-    __bf16* __restrict__ dq, int q0, int cnt, int H, int Skv, int K, int q_start) {
+    __bf16* __restrict__ dq, int q0, int cnt, int H, int Skv, int K, int q_start, const int* __restrict__ dup_flag) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int STAGE_BYTES = TILE_BYTES + PDS_KIND_BYTES;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -353,6 +353,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
     }
   }
   // ---- write dQ: accumulator e of a lane is d = 32*dt + 8*(e/4) + 4*g + (e%4), head = 32*hg + r ----
+  const bool poison = *dup_flag != 0;          // a query row with a repeated id: NaN instead of a sum that misses a term
 #pragma unroll
   for (int u = 0; u < 9; u++) {
     if (u < 8) mfma_done_a(acc[u]); else mfma_done_v(acc[u]);
@@ -363,6 +364,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
       unsigned short* op = (unsigned short*)dq + ((size_t)qi * H + h) * DQK + 32 * dt + 8 * g;
       uint4 o[2];
       acc_row_to_16B(acc[u], 1.0f, o);
+      if (poison) o[0] = o[1] = make_uint4(0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u);
       *(uint4*)op = o[0];
       *(uint4*)(op + 16) = o[1];
     }
@@ -635,9 +637,12 @@ __global__ __launch_bounds__(288) void bwd_reduce_kernel(const unsigned char* __
   }
 }
 
-__global__ void cast_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dstp, size_t n) {
+// fp32 accumulator -> bf16 dKV; NaN everywhere when a query row held a repeated id
+__global__ void cast_bf16_kernel(const float* __restrict__ src, unsigned short* __restrict__ dstp, size_t n,
+                                 const int* __restrict__ dup_flag) {
+  const bool poison = *dup_flag != 0;
   for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x)
-    dstp[e] = f32_to_bf16_bits(src[e]);
+    dstp[e] = poison ? (unsigned short)0x7fc0 : f32_to_bf16_bits(src[e]);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -646,7 +651,7 @@ __global__ void cast_bf16_kernel(const float* __restrict__ src, unsigned short* 
 struct BwdPlan {
   int chunk;            // queries per pass over the buffers
   int W;                // bitmap words per key
-  size_t off_bitmap, off_prefix, off_count, off_start, off_dst, off_sorted, off_pds, off_rows, off_acc, total;
+  size_t off_bitmap, off_prefix, off_count, off_start, off_flag, off_dst, off_sorted, off_pds, off_rows, off_acc, total;
 };
 
 size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -660,6 +665,7 @@ BwdPlan layout_plan(int chunk, int Skv, int K) {
   p.off_prefix = o; o = align_up(o + order::prefix_words(chunk, Skv) * 4);
   p.off_count = o; o = align_up(o + (size_t)(Skv + 1) * 4);
   p.off_start = o; o = align_up(o + (size_t)(Skv + 1) * 4);
+  p.off_flag = o; o = align_up(o + 4);
   p.off_dst = o; o = align_up(o + (size_t)chunk * K * 4);
   p.off_sorted = o; o = align_up(o + (size_t)chunk * K * 4);
   p.off_pds = o; o = align_up(o + (size_t)chunk * (K / BI) * PDS_TILE_BYTES);
@@ -714,6 +720,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   unsigned* prefix = (unsigned*)(ws + p.off_prefix);
   int* count = (int*)(ws + p.off_count);
   int* start = (int*)(ws + p.off_start);
+  int* dup_flag = (int*)(ws + p.off_flag);
   int* dstp = (int*)(ws + p.off_dst);
   int* sorted = (int*)(ws + p.off_sorted);
   unsigned char* pds = ws + p.off_pds;
@@ -737,6 +744,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   }
 #define DSA_MARK(i) do { if (pass_ms) hipEventRecord(ev[i], st); } while (0)
   bool first = true;
+  order::clear_flag(dup_flag, st);
   for (int q0 = 0; q0 < S; q0 += p.chunk) {
     const int cnt = S - q0 < p.chunk ? S - q0 : p.chunk;
     DSA_MARK(0);
@@ -746,7 +754,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     // (The list is put together in LDS next to a bitmap over all keys; with more keys than fit there the
     // passes walk the caller's slot order instead.)
     const bool sort_ids = order::sorted_list_fits(Skv, K);
-    order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st, sort_ids ? sorted : nullptr);
+    order::build(ids, q0, cnt, K, Skv, q_start, bitmap, prefix, count, start, dstp, p.W, st, dup_flag, sort_ids ? sorted : nullptr);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
     const int* sids = sort_ids ? sorted : ids + (size_t)q0 * K;      // row ql belongs to query q0 + ql
     DSA_MARK(1);
@@ -754,7 +762,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
                                                           (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(P, dS)");
     DSA_MARK(2);
-    bwd_dq_kernel<3><<<dim3(cnt), dim3(512), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start);
+    bwd_dq_kernel<3><<<dim3(cnt), dim3(512), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start, dup_flag);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ)");
     DSA_MARK(3);
     bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, sids, pds, dstp, rows, q0, cnt,
@@ -773,7 +781,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   if (S == 0) {
     order::zero_u32_kernel<<<dim3(256), dim3(256), 0, st>>>((unsigned*)acc, (size_t)Skv * DQK);
   }
-  cast_bf16_kernel<<<dim3(2048), dim3(256), 0, st>>>(acc, (unsigned short*)dkv, (size_t)Skv * DQK);
+  cast_bf16_kernel<<<dim3(2048), dim3(256), 0, st>>>(acc, (unsigned short*)dkv, (size_t)Skv * DQK, dup_flag);
   DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(cast)");
   (void)NT;
   if (pass_ms) for (int i = 0; i < 6; i++) hipEventDestroy(ev[i]);

@@ -2,7 +2,10 @@
 // work only (bitmap key x query, row-wise prefix popcounts, exclusive scan over keys), so it is
 // identical from run to run.  Used by the deterministic scatter-accumulations of the backward
 // kernels: pair (q, slot) with key v gets row  start[v] + #{q' < q : q' selects v}.
-// Ids within one query row must be distinct (any top-k guarantees it).
+// Ids within one query row must be distinct (any top-k guarantees it): a repeated id has one bit and
+// one row like any other, so one of its contributions would be lost.  The first kernel notices a
+// repeated id (the bit it sets is set already) and raises *dup_flag; the callers' last kernels then
+// fill their outputs with NaN instead of returning sums that silently miss a term.
 #pragma once
 #include "dsa_common.h"
 
@@ -21,7 +24,7 @@ static __global__ void zero_u32_kernel(unsigned* __restrict__ p, size_t n) {
 // bytes.
 static __global__ __launch_bounds__(256) void qmap_kernel(const int* __restrict__ ids, int q0, int cnt, int K, int Skv,
                                                           int q_start, unsigned* __restrict__ qmap, int Wk,
-                                                          int* __restrict__ sorted) {
+                                                          int* __restrict__ sorted, int* __restrict__ dup_flag) {
   extern __shared__ unsigned qbits[];        // Wk words; with `sorted`, Wk more for the prefix counts and K for the list
   __shared__ int wave_tot[4];
   const int ql = blockIdx.x;
@@ -33,7 +36,10 @@ static __global__ __launch_bounds__(256) void qmap_kernel(const int* __restrict_
     for (int i = 0; i < 8; i++) v[i] = t0 + i * 256 < K ? ids[(size_t)(q0 + ql) * K + t0 + i * 256] : -1;
 #pragma unroll
     for (int i = 0; i < 8; i++)
-      if (v[i] >= 0 && v[i] < Skv && v[i] <= q_start + q0 + ql) atomicOr(&qbits[v[i] >> 5], 1u << (v[i] & 31));
+      if (v[i] >= 0 && v[i] < Skv && v[i] <= q_start + q0 + ql) {
+        const unsigned bit = 1u << (v[i] & 31);
+        if (atomicOr(&qbits[v[i] >> 5], bit) & bit) *dup_flag = 1;      // every writer stores the same value
+      }
   }
   __syncthreads();
   for (int w = threadIdx.x; w < Wk; w += 256) qmap[(size_t)ql * Wk + w] = qbits[w];
@@ -171,14 +177,16 @@ constexpr int MAX_KEYS = 150 * 1024 * 8;
 inline bool sorted_list_fits(int Skv, int K) {
   return (size_t)((Skv + 31) / 32) * 8 + (size_t)K * 4 <= (size_t)150 * 1024;
 }
+// dup_flag: one int the caller has cleared (clear_flag) before the first block of queries of a call.
+inline void clear_flag(int* dup_flag, hipStream_t st) { zero_u32_kernel<<<dim3(1), dim3(64), 0, st>>>((unsigned*)dup_flag, 1); }
 inline void build(const int* ids, int q0, int cnt, int K, int Skv, int q_start, unsigned* bitmap, unsigned* prefix,
-                  int* count, int* start, int* dst, int W, hipStream_t st, int* sorted = nullptr) {
+                  int* count, int* start, int* dst, int W, hipStream_t st, int* dup_flag, int* sorted = nullptr) {
   const int Wk = (Skv + 31) / 32;
   unsigned* qmap = prefix;
   const size_t lds = (size_t)Wk * 4 * (sorted ? 2 : 1) + (sorted ? (size_t)K * 4 : 0);
   if (lds > 48 * 1024)
     (void)hipFuncSetAttribute((const void*)qmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  qmap_kernel<<<dim3(cnt), dim3(256), lds, st>>>(ids, q0, cnt, K, Skv, q_start, qmap, Wk, sorted);
+  qmap_kernel<<<dim3(cnt), dim3(256), lds, st>>>(ids, q0, cnt, K, Skv, q_start, qmap, Wk, sorted, dup_flag);
   // every word of the bitmap is written (zeros beyond the last query), so no clearing pass is needed
   bm_transpose_kernel<<<dim3((W + 7) / 8, Wk), dim3(256), 0, st>>>(qmap, cnt, Skv, Wk, bitmap, W);
   bm_prefix_kernel<<<dim3((Skv + 3) / 4), dim3(256), 0, st>>>(bitmap, prefix, count, Skv, W);

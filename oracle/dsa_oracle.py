@@ -208,7 +208,7 @@ def sparse_mla_valid(idx: torch.Tensor, s_kv: int, q_start: int) -> torch.Tensor
     dsa_fused_kernels.py:2051 ("invalid indices should be set to -1 or numbers >= s_kv").
     """
     sq = idx.shape[0]
-    pos = torch.arange(sq, dtype=torch.int64).unsqueeze(-1) + int(q_start)
+    pos = torch.arange(sq, dtype=torch.int64, device=idx.device).unsqueeze(-1) + int(q_start)
     i64 = idx.to(torch.int64)
     return (i64 >= 0) & (i64 < s_kv) & (i64 <= pos)
 
@@ -274,6 +274,75 @@ def sparse_mla_bwd(q, kv, idx, dout, q_start=0, sm_scale=None, d_v=512, dtype=to
     out, _, _ = sparse_mla_fwd(qd, kvd, idx, q_start, sm_scale, d_v, dtype=dtype, attn_sink=attn_sink)
     out.backward(dout.to(dtype))
     return qd.grad, kvd.grad
+
+
+def sparse_mla_bwd_kernel_rounding(q, kv, idx, dout, q_start=0, sm_scale=None, d_v=512, out=None, lse=None,
+                                   round_p_ds_bf16=True, round_rows_bf16=False, return_abs_sum=False, chunk=32,
+                                   attn_sink=None, dtype=torch.float32):
+    """dQ, dKV by the closed form of the reference's backward kernel, with that kernel's rounding
+    points (ops/tilelang_ops/sparse_mla_bwd.py): every product accumulates in fp32 from bf16
+    operands; ``P = exp(S*scale - lse)`` (:192-193) and ``dS = P*(dP - Delta)*scale`` (:197-199,
+    from the fp32 P) are each cast to bf16 (``P_shared_cast``, ``dP_shared_cast``: :194, :200)
+    before they enter ``dQ = dS.KV`` (:201-202) and ``dKV[idx] += dS^T.Q + P^T.dO`` (:203-209);
+    dKV is accumulated in fp32 (atomic adds of the fp32 tile, :210-227).  ``Delta = rowsum(O*dO)``
+    (preprocess kernel, :26-43) uses the forward's output as stored (bf16) and ``lse`` is the
+    forward's; both default to this oracle's fp32 forward with the output rounded to bf16.  With ``round_p_ds_bf16=False`` this is the same closed form in fp32,
+    which must agree with autograd (:func:`sparse_mla_bwd`).  Returns fp32 ``(dQ, dKV)``.
+    ``round_rows_bf16`` adds the one rounding the HIP build has on top of the reference kernel's:
+    the contribution of a (query, key) pair to dKV - the sum over all heads, one row of 576 values
+    - is rounded to bf16 before the rows of a key are summed in fp32.  ``return_abs_sum`` also
+    returns ``A[key, d] = sum over pairs |row[d]|`` and ``M[key, d] = max over pairs |row[d]|``:
+    ``2**-9 * A`` bounds what that rounding can change (round-to-nearest bf16 moves a value by at
+    most 2**-9 of its size), and ``2**-7 * M`` is one step of the bf16 grid at the largest row, i.e.
+    what two evaluations differ by when that row lands on either side of a rounding boundary.
+    Written with device-agnostic tensor ops, so a test may evaluate it on tensors that live on
+    the GPU when the full benchmark sizes are too slow for the host (it stays a torch fp32
+    evaluation of the same lines either way).  ``attn_sink`` only enters through ``lse`` (the sink
+    is one more term of the softmax denominator and has no value row), i.e. through the default
+    forward when ``lse`` is not given.  ``dtype`` is the arithmetic between the rounding points:
+    fp32 as in the kernel, or fp64, which makes the result independent of the host's summation
+    order (an fp32 sum that lands on the other side of a bf16 rounding boundary on another CPU
+    would move a term by 2**-8 of its size).
+    """
+    sq, h, dqk = q.shape
+    skv = kv.shape[0]
+    if sm_scale is None:
+        sm_scale = dqk ** -0.5
+    if out is None or lse is None:
+        o32, l32, _ = sparse_mla_fwd(q, kv, idx, q_start, sm_scale, d_v, attn_sink=attn_sink)
+        out = o32.to(torch.bfloat16) if out is None else out
+        lse = l32 if lse is None else lse
+    valid = sparse_mla_valid(idx, skv, q_start)
+    safe = torch.where(valid, idx.to(torch.int64), torch.zeros_like(idx, dtype=torch.int64))
+    qf, kvf, dof = q.to(dtype), kv.to(dtype), dout.to(dtype)
+    delta = (out.to(dtype) * dof).sum(-1)                                # [sq, h]
+    lse_f = torch.where(torch.isinf(lse), torch.zeros_like(lse), lse).to(dtype)
+    dq = torch.zeros(sq, h, dqk, device=q.device, dtype=dtype)
+    dkv = torch.zeros(skv, dqk, device=q.device, dtype=dtype)
+    abs_sum = torch.zeros(skv, dqk, device=q.device, dtype=dtype) if return_abs_sum else None
+    abs_max = torch.zeros(skv, dqk, device=q.device, dtype=dtype) if return_abs_sum else None
+    rnd = (lambda t: t.to(torch.bfloat16).to(dtype)) if round_p_ds_bf16 else (lambda t: t)
+    for s in range(0, sq, chunk):
+        e = min(sq, s + chunk)
+        kvg = kvf[safe[s:e]]                                             # [c, K, dqk]
+        sc = torch.einsum("mhd,mkd->mhk", qf[s:e], kvg)
+        p = torch.exp(sc * sm_scale - lse_f[s:e].unsqueeze(-1))
+        p = p.masked_fill(~valid[s:e].unsqueeze(1), 0.0)
+        dp = torch.einsum("mhd,mkd->mhk", dof[s:e], kvg[..., :d_v])
+        ds = p * (dp - delta[s:e].unsqueeze(-1)) * sm_scale
+        p_b, ds_b = rnd(p), rnd(ds)
+        dq[s:e] = torch.einsum("mhk,mkd->mhd", ds_b, kvg)
+        contrib = torch.einsum("mhk,mhd->mkd", ds_b, qf[s:e])
+        contrib[..., :d_v] += torch.einsum("mhk,mhd->mkd", p_b, dof[s:e])
+        if round_rows_bf16:
+            contrib = contrib.to(torch.bfloat16).to(dtype)
+        dkv.index_add_(0, safe[s:e].reshape(-1), contrib.reshape(-1, dqk))   # invalid slots add zeros to row 0
+        if return_abs_sum:
+            abs_sum.index_add_(0, safe[s:e].reshape(-1), contrib.abs().reshape(-1, dqk))
+            abs_max.scatter_reduce_(0, safe[s:e].reshape(-1, 1).expand(-1, dqk), contrib.abs().reshape(-1, dqk), "amax")
+    if return_abs_sum:
+        return dq, dkv, abs_sum, abs_max
+    return dq, dkv
 
 
 # --------------------------------------------------------------------------------------------

@@ -33,7 +33,12 @@ def mla_golden():
     out, lse, p_out = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, c["q_start"], inp.sm_scale, 512, dtype=torch.float64)
     dq, dkv = O.sparse_mla_bwd(inp.q, inp.kv, inp.idx, inp.dout, c["q_start"], inp.sm_scale, 512, dtype=torch.float64)
     tgt = O.attn_dist(p_out.float(), inp.sm_scale)
+    # dKV with the rounding points of the HIP backward (bf16 P / dS as in the reference kernel, bf16
+    # per-pair rows), fp32 evaluation
+    _, dkv_r = O.sparse_mla_bwd_kernel_rounding(inp.q, inp.kv, inp.idx, inp.dout, c["q_start"], inp.sm_scale, 512,
+                                                round_rows_bf16=True, dtype=torch.float64)
     return dict(out=sample(out, 5, 3, 37), lse=sample(lse, 1, 1), dq=sample(dq, 5, 3, 41), dkv=sample(dkv, 3, 29),
+                dkv_kernel_rounding=sample(dkv_r, 3, 29),
                 target=sample(tgt, 7, 5), sums=np.array([out.sum().item(), lse.sum().item(), dq.abs().sum().item(),
                                                           dkv.abs().sum().item()]))
 

@@ -41,7 +41,10 @@ def test_kernels_match_mla_fixture(gpu):
     inp = O.make_mla_inputs(c["S"], c["H"], c["K"], seed=c["seed"], skv=c["skv"], q_start=c["q_start"])
     q, kv, idx, do = inp.q.to(gpu), inp.kv.to(gpu), inp.idx.to(gpu), inp.dout.to(gpu)
     out, lse, p = ops.sparse_mla_fwd(q, kv, idx, c["q_start"], inp.sm_scale, 512, True, torch.float32)
-    dq, dkv = ops.sparse_mla_bwd(q, kv, out, do, idx, lse, c["q_start"], inp.sm_scale)
+    # the backward takes the forward's out and lse as inputs (Delta = rowsum(out * dO) feels every bf16
+    # rounding of out): hand it the ones the fixture was made with, the oracle's
+    o_ref, l_ref, _ = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, c["q_start"], inp.sm_scale, 512)
+    dq, dkv = ops.sparse_mla_bwd(q, kv, o_ref.to(torch.bfloat16).to(gpu), do, idx, l_ref.to(gpu), c["q_start"], inp.sm_scale)
     tgt = ops.attn_dist(p, inp.sm_scale)
 
     def close(got, want, atol, rtol=1e-2):
@@ -50,8 +53,12 @@ def test_kernels_match_mla_fixture(gpu):
     close(G.sample(out.cpu(), 5, 3, 37), ref["out"], 2e-2)
     close(G.sample(lse.cpu(), 1, 1), ref["lse"], 1e-4, 0)
     close(G.sample(tgt.cpu(), 7, 5), ref["target"], 1e-5, 1e-3)
-    close(G.sample(dq.cpu(), 5, 3, 41), ref["dq"], max(2e-2, 5e-3 * np.abs(ref["dq"]).max()))
-    close(G.sample(dkv.cpu(), 3, 29), ref["dkv"], max(2e-2, 5e-3 * np.abs(ref["dkv"]).max()))
+    close(G.sample(dq.cpu(), 5, 3, 41), ref["dq"], 2e-2)
+    # dKV element by element against the oracle evaluated with the kernels' rounding points; the plain
+    # fp64 gradient is out of reach of any bf16-operand backward by the margin recorded in gpu_util
+    from tests.gpu_util import FP32_DKV_EXCESS_LIMIT
+    close(G.sample(dkv.cpu(), 3, 29), ref["dkv_kernel_rounding"], 2e-2)
+    close(G.sample(dkv.cpu(), 3, 29), ref["dkv"], 2e-2 + FP32_DKV_EXCESS_LIMIT)
 
 
 @pytest.mark.gpu

@@ -8,7 +8,7 @@ import torch
 
 from oracle import csa_oracle as C
 from oracle import dsa_oracle as O
-from tests.gpu_util import assert_close
+from tests.gpu_util import FP32_DKV_EXCESS_LIMIT, FP32_DQ_EXCESS_LIMIT, assert_close, assert_mla_grads
 
 pytestmark = pytest.mark.gpu
 
@@ -140,5 +140,11 @@ def test_window_plus_compressed_attention_equals_dense_masked_attention(gpu):
     assert out.shape == (1, sq, H, 512)
     assert_close(out[0], ref, "out")
     out.backward(dout.to(gpu).unsqueeze(0))
-    assert_close(qg.grad, qd.grad, "dq", scale_aware=True)
-    assert_close(kg.grad, kd.grad, "dkv", scale_aware=True)
+    # gradients: element by element against the oracle with the kernels' rounding points, then the distance
+    # from the dense fp64 gradients, which a bf16-operand backward cannot bring under the elementwise bound
+    d = (qg.grad.float().cpu().double() - qd.grad).abs() - (2e-2 + 1e-2 * qd.grad.abs())
+    assert d.max().item() <= FP32_DQ_EXCESS_LIMIT
+    assert_mla_grads(qg.grad, kg.grad, q, kv_full, ids[0].int(), dout, kv_full.shape[0], sm_scale, attn_sink=sink,
+                     out=out[0])
+    d = (kg.grad.float().cpu().double() - kd.grad).abs() - (2e-2 + 1e-2 * kd.grad.abs())
+    assert d.max().item() <= FP32_DKV_EXCESS_LIMIT

@@ -49,6 +49,19 @@ def test_indexer_bwd_against_oracle(gpu, S, Hi, K, seed):
     assert ew.max().item() <= 1e-4 * rw.abs().max().item()
 
 
+def test_indexer_bwd_with_a_repeated_id_returns_nan_keys(gpu):
+    from loongforge_amd import ops
+
+    iq, ik, w = O.make_indexer_inputs(256, 64, 128, seed=5)
+    _, idx, aux = O.indexer_forward(iq, ik, w, 128, 0, None)
+    idx = idx.clone()
+    idx[200, 3] = idx[200, 17]
+    g = torch.ones(256, 128)
+    dq, dk, dw = ops.indexer_bwd(g.to(gpu), aux["q8"].to(gpu), aux["k8"].to(gpu), aux["k_scale"].to(gpu),
+                                 aux["weight_scaled"].to(gpu).contiguous(), idx.to(gpu))
+    assert torch.isnan(dk).all()
+
+
 def test_indexer_kernel_module_forward_and_backward(gpu):
     """DSAIndexerKernel with the reference's call signature: unpadded head count / head dim (the
     reference's own CPU-sized configuration uses 4 heads of dim 64), packed documents, autograd."""

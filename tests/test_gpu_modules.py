@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import dsa_oracle as O
-from tests.gpu_util import assert_close
+from tests.gpu_util import assert_close, assert_mla_grads
 
 pytestmark = pytest.mark.gpu
 
@@ -34,9 +34,7 @@ def test_dot_product_attention_layouts_and_autograd(gpu):
     assert_close(out[0], ro, "out")
     assert torch.isinf(p_out[:, :, 100:]).all()
     out.backward(inp.dout.to(gpu).unsqueeze(0))
-    rdq, rdkv = O.sparse_mla_bwd(inp.q, inp.kv, inp.idx, inp.dout, 0, inp.sm_scale, 512)
-    assert_close(q.grad, rdq, "dq", scale_aware=True)
-    assert_close(kv.grad, rdkv, "dkv", scale_aware=True)
+    assert_mla_grads(q.grad, kv.grad, inp.q, inp.kv, inp.idx, inp.dout, 0, inp.sm_scale, out=out[0])
     # thd: query [t, h, d], kv [t, d], ids handed as [1, t, topk]
     psp = PackedSeqParams(qkv_format="thd")
     out2 = attn(inp.q.to(gpu), inp.kv.to(gpu), ids.unsqueeze(0), 0, None, packed_seq_params=psp)
@@ -61,9 +59,11 @@ def test_dot_product_attention_layouts_and_autograd(gpu):
     ro3, _, _ = O.sparse_mla_fwd(inp.q, inp.kv, cut, 0, inp.sm_scale, 512, attn_sink=sink_h)
     assert_close(out3[0], ro3, "out with topk_length and sink")
     out3.backward(inp.dout.to(gpu).unsqueeze(0))
-    rdq3, rdkv3 = O.sparse_mla_bwd(inp.q, inp.kv, cut, inp.dout, 0, inp.sm_scale, 512, attn_sink=sink_h)
-    assert_close(q.grad, rdq3, "dq with topk_length and sink", scale_aware=True)
-    assert_close(kv.grad, rdkv3, "dkv with topk_length and sink", scale_aware=True)
+    from loongforge_amd import ops
+    cut_pad = torch.nn.functional.pad(cut, (0, 28), value=-1).to(gpu)          # the module pads top-k 100 to 128
+    _, lse3, _ = ops.sparse_mla_fwd(q.detach(), kv.detach(), cut_pad, 0, inp.sm_scale, attn_sink=sink_h.to(gpu))
+    assert_mla_grads(q.grad, kv.grad, inp.q, inp.kv, cut, inp.dout, 0, inp.sm_scale, "topk_length and sink:", attn_sink=sink_h,
+                     out=out3[0], lse=lse3)
 
 
 def test_sparse_mla_bwd_interface_signature(gpu):
@@ -77,9 +77,7 @@ def test_sparse_mla_bwd_interface_signature(gpu):
     dq, dkv = sparse_mla_bwd_interface(q, kv.unsqueeze(1), out, do, idx.unsqueeze(1), lse, offsets, chunk_offset=30,
                                        sm_scale=inp.sm_scale)
     assert dq.shape == q.shape and dkv.shape == (200, 1, 576)
-    rdq, rdkv = O.sparse_mla_bwd(inp.q, inp.kv, inp.idx, inp.dout, 30, inp.sm_scale, 512)
-    assert_close(dq, rdq, "dq", scale_aware=True)
-    assert_close(dkv[:, 0], rdkv, "dkv", scale_aware=True)
+    assert_mla_grads(dq, dkv[:, 0], inp.q, inp.kv, inp.idx, inp.dout, 30, inp.sm_scale, out=out, lse=lse)
 
 
 class _Linear(torch.nn.Module):
@@ -145,10 +143,8 @@ def test_fused_attention_module_matches_oracle_pipeline(gpu):
 
     dout = torch.randn(1, S, H, 512, generator=g).to(torch.bfloat16).to(gpu)
     out.backward(dout)
-    rdq, rdkv = O.sparse_mla_bwd(query.detach().cpu()[:, 0], key.detach().cpu()[:, 0], ref["idx"], dout[0].cpu(), 0,
-                                 mod.softmax_scale, 512)
-    assert_close(query.grad[:, 0], rdq, "dq", scale_aware=True)
-    assert_close(key.grad[:, 0], rdkv, "dkv", scale_aware=True)
+    assert_mla_grads(query.grad[:, 0], key.grad[:, 0], query.detach().cpu()[:, 0], key.detach().cpu()[:, 0], ref["idx"],
+                     dout[0].cpu(), 0, mod.softmax_scale, out=out[0])
     # the indexer loss reached the indexer's weights and only those
     grads = {n: p.grad for n, p in mod.named_parameters()}
     assert all(gv is not None and torch.isfinite(gv).all() and gv.abs().max() > 0 for n, gv in grads.items()

@@ -181,6 +181,62 @@ def test_bwd_closed_form_matches_autograd_and_dS_sums_to_zero():
     torch.testing.assert_close(dkv, dkv_ref, rtol=1e-9, atol=1e-12)
 
 
+def test_bwd_kernel_rounding_form_without_rounding_equals_autograd():
+    sq, h, dqk, dv, K = 24, 4, 32, 16, 8
+    q, kv, idx = _inputs(sq, h, K, dqk, seed=41, dtype=torch.float32)
+    dout = torch.randn(sq, h, dv, generator=torch.Generator().manual_seed(43))
+    out, lse, _ = O.sparse_mla_fwd(q, kv, idx, 0, 0.3, dv)
+    dq, dkv = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, dout, 0, 0.3, dv, out=out, lse=lse, round_p_ds_bf16=False)
+    rdq, rdkv = O.sparse_mla_bwd(q, kv, idx, dout, 0, 0.3, dv)
+    torch.testing.assert_close(dq, rdq, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(dkv, rdkv, rtol=1e-4, atol=1e-5)
+
+
+def test_bwd_kernel_rounding_form_matches_loops_with_bf16_casts():
+    # the reference kernel's rounding points (ops/tilelang_ops/sparse_mla_bwd.py:192-209) written out
+    # as loops over (query, head, slot) in fp64, the two casts done per element
+    sq, h, dqk, dv, K = 9, 2, 16, 8, 4
+    g = torch.Generator().manual_seed(47)
+    q = torch.randn(sq, h, dqk, generator=g).to(torch.bfloat16)
+    kv = torch.randn(sq, dqk, generator=g).to(torch.bfloat16)
+    dout = torch.randn(sq, h, dv, generator=g).to(torch.bfloat16)
+    idx = O.causal_random_topk_indices(sq, K, 48)
+    idx[3, 1] = -1
+    sm = 0.29
+    o32, lse, _ = O.sparse_mla_fwd(q, kv, idx, 0, sm, dv)
+    out = o32.to(torch.bfloat16)
+    dq, dkv = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, dout, 0, sm, dv, out=out, lse=lse)
+    bf = lambda x: torch.tensor(x, dtype=torch.float32).to(torch.bfloat16).double().item()
+    qd, kd, dd, od = q.double(), kv.double(), dout.double(), out.double()
+    dq_ref, dkv_ref = torch.zeros(sq, h, dqk, dtype=torch.float64), torch.zeros(sq, dqk, dtype=torch.float64)
+    n_changed = 0
+    for i in range(sq):
+        for hh in range(h):
+            delta = (od[i, hh] * dd[i, hh]).sum().item()
+            for t in range(K):
+                j = int(idx[i, t])
+                if j < 0 or j > i:
+                    continue
+                p = math.exp((qd[i, hh] * kd[j]).sum().item() * sm - lse[i, hh].item())
+                dp = (dd[i, hh] * kd[j, :dv]).sum().item()
+                ds = p * (dp - delta) * sm
+                pb, dsb = bf(p), bf(ds)
+                n_changed += (pb != p) + (dsb != ds)
+                dq_ref[i, hh] += dsb * kd[j]
+                dkv_ref[j] += dsb * qd[i, hh]
+                dkv_ref[j, :dv] += pb * dd[i, hh]
+    assert n_changed > 50                      # the casts are not no-ops on this input
+    # fp32 evaluation of exp / products may flip a bf16 rounding of P or dS by one ulp (2^-8
+    # relative) now and then; sums of a handful of such terms stay within a few 1e-3 of the loops
+    torch.testing.assert_close(dq.double(), dq_ref, rtol=0, atol=4e-3 * dq_ref.abs().max().item())
+    torch.testing.assert_close(dkv.double(), dkv_ref, rtol=0, atol=4e-3 * dkv_ref.abs().max().item())
+    # and the rounding is visible: the fp32 closed form differs from the rounded one
+    dq32, dkv32 = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, dout, 0, sm, dv, out=out, lse=lse, round_p_ds_bf16=False)
+    assert (dkv32 - dkv).abs().max() > 1e-4
+    # median agreement with the loops is at fp32 level (the casts land on the same bf16 values)
+    assert (dkv.double() - dkv_ref).abs().median().item() <= 1e-5 * dkv_ref.abs().max().item()
+
+
 def test_bwd_gradcheck_fp64():
     sq, h, dqk, dv, K = 6, 2, 8, 4, 3
     q, kv, idx = _inputs(sq, h, K, dqk, seed=19)
