@@ -105,6 +105,21 @@ int dsa_indexer_topk_fwd(const void* q8, const float* q_w, const void* k8, const
                          size_t workspace_bytes, void* stream);
 
 /*
+ * dsa_indexer_topk_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same inputs, outputs and results, no
+ * workspace argument.  The logits blocks live in a 64 MiB device array inside the library, which every
+ * GPU the library runs on holds until the process ends; at most 65536 keys (a block of 256 queries
+ * must fit), more is refused with DSA_ERR_BAD_ARG.  The call allocates nothing; calls that overlap on
+ * one GPU share the array and race, so order them on one stream.  The first call on a device looks
+ * up the array's address there (not a stream operation: make it outside a graph capture).
+ * No counterpart in the reference, whose wrapper lets torch allocate the logits
+ * (dsa_fused_kernels.py:2366-2380).
+ */
+int dsa_indexer_topk_fwd_static(const void* q8, const float* q_w, const void* k8, const float* k_scale,
+                                const int32_t* ks, const int32_t* ke, int S, int Hi, int Sk, int K,
+                                int sorted, float* scores, int32_t* ids, void* stream);
+
+/*
  * Sparse gradients of the selected logits w.r.t. the fp8 payloads and the scaled weights
  * (scales are constants):  with j = ids[i,t] >= 0, r_h = q8[i,h,:] . k8[j,:],
  *   d_qw[i,h]   = sum_t g[i,t] k_scale[j] relu(r_h)

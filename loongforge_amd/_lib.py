@@ -23,6 +23,7 @@ SIGNATURES = {
     "dsa_topk": (_i, [_vp, _i, _i64, _vp, _vp, _i, _vp, _i, _i, _vp, _vp, _vp]),
     "dsa_indexer_topk_workspace_bytes": (_sz, [_i, _i, _i]),
     "dsa_indexer_topk_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _sz, _vp]),
+    "dsa_indexer_topk_fwd_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "dsa_indexer_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "dsa_indexer_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
     "dsa_sparse_mla_fwd": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _i, _vp]),

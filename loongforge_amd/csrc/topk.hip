@@ -529,16 +529,10 @@ extern "C" size_t dsa_indexer_topk_workspace_bytes(int S, int Sk, int K) {
   return (size_t)rows * (size_t)Sk * 4;
 }
 
-extern "C" int dsa_indexer_topk_fwd(const void* q8, const float* q_w, const void* k8, const float* k_scale,
-                                    const int32_t* ks, const int32_t* ke, int S, int Hi, int Sk, int K, int sorted,
-                                    float* scores, int32_t* ids, void* workspace, size_t workspace_bytes,
-                                    void* stream) {
-  hipStream_t st = (hipStream_t)stream;
-  if (S == 0) return DSA_OK;
-  DSA_REQUIRE(workspace != nullptr && workspace_bytes >= dsa_indexer_topk_workspace_bytes(S, Sk, K),
-              "dsa_indexer_topk_fwd: workspace of %zu bytes is too small", workspace_bytes);
-  int rows = fused_block_rows(Sk);
-  float* lg = (float*)workspace;
+// Logits of `rows` queries at a time into lg ([rows][Sk] floats), then their top-k.
+static int indexer_topk_blocks(const void* q8, const float* q_w, const void* k8, const float* k_scale, const int32_t* ks,
+                               const int32_t* ke, int S, int Hi, int Sk, int K, int sorted, float* scores, int32_t* ids,
+                               float* lg, int rows, hipStream_t st) {
   for (int q0 = 0; q0 < S; q0 += rows) {
     const int cnt = S - q0 < rows ? S - q0 : rows;
     int rc = dsa_indexer_logits_block(q8, q_w, k8, k_scale, ks, ke, S, Hi, Sk, lg, Sk, Sk, 0, 0, q0, cnt, st);
@@ -548,4 +542,57 @@ extern "C" int dsa_indexer_topk_fwd(const void* q8, const float* q_w, const void
     if (rc != DSA_OK) return rc;
   }
   return DSA_OK;
+}
+
+extern "C" int dsa_indexer_topk_fwd(const void* q8, const float* q_w, const void* k8, const float* k_scale,
+                                    const int32_t* ks, const int32_t* ke, int S, int Hi, int Sk, int K, int sorted,
+                                    float* scores, int32_t* ids, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
+  if (S == 0) return DSA_OK;
+  DSA_REQUIRE(workspace != nullptr && workspace_bytes >= dsa_indexer_topk_workspace_bytes(S, Sk, K),
+              "dsa_indexer_topk_fwd: workspace of %zu bytes is too small", workspace_bytes);
+  return indexer_topk_blocks(q8, q_w, k8, k_scale, ks, ke, S, Hi, Sk, K, sorted, scores, ids, (float*)workspace,
+                             fused_block_rows(Sk), (hipStream_t)stream);
+}
+
+// ---- the same without any allocation by anyone: the logits blocks live in a device array of the library ----
+// For callers that cannot allocate device memory (code under HIP graph capture, tight serving loops):
+// they pass inputs and outputs only.  Every GPU the library runs on holds its own copy of the array
+// until the process ends; calls that overlap on one GPU share it and race - order them on one stream.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)64 << 20;
+constexpr int STATIC_MIN_ROWS = 256;           // a block of fewer queries would leave most compute units idle
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+#include <mutex>
+static std::mutex scratch_mutex;
+static void* scratch_ptr[64];                  // per device: the array's address on that device (0 = not asked yet)
+
+extern "C" int dsa_indexer_topk_fwd_static(const void* q8, const float* q_w, const void* k8, const float* k_scale,
+                                           const int32_t* ks, const int32_t* ke, int S, int Hi, int Sk, int K,
+                                           int sorted, float* scores, int32_t* ids, void* stream) {
+  if (S == 0) return DSA_OK;
+  DSA_REQUIRE(Sk > 0 && (size_t)Sk * 4 * STATIC_MIN_ROWS <= STATIC_SCRATCH_BYTES,
+              "dsa_indexer_topk_fwd_static: at most %zu keys fit the library's %zu MiB scratch array, got %d "
+              "(use dsa_indexer_topk_fwd with a workspace)",
+              STATIC_SCRATCH_BYTES / (4 * STATIC_MIN_ROWS), STATIC_SCRATCH_BYTES >> 20, Sk);
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    DSA_FAIL(DSA_ERR_LAUNCH, "dsa_indexer_topk_fwd_static: no current device");
+  void* base;
+  {
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {         // first call on this device: the array's address here
+      void* p = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || p == nullptr)
+        DSA_FAIL(DSA_ERR_LAUNCH, "dsa_indexer_topk_fwd_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+      scratch_ptr[dev] = p;
+    }
+    base = scratch_ptr[dev];
+  }
+  int rows = (int)(STATIC_SCRATCH_BYTES / ((size_t)Sk * 4)) / 8 * 8;
+  // (nothing in the array has to start at zero: the logits kernel writes columns [ks, ke) of every row of a block
+  // and the selection reads no others)
+  return indexer_topk_blocks(q8, q_w, k8, k_scale, ks, ke, S, Hi, Sk, K, sorted, scores, ids, (float*)base, rows,
+                             (hipStream_t)stream);
 }
