@@ -46,18 +46,6 @@ DSA_MFMA_FN(mfma_a_av, "a", "a", "v")
 __device__ __forceinline__ void mfma_done_v(f32x16& acc) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(acc)); }
 __device__ __forceinline__ void mfma_done_a(f32x16& acc) { asm volatile("s_nop 15\n\ts_nop 3" : "+a"(acc)); }
 
-// vmcnt wait with a run-time bound (the instruction needs an immediate)
-__device__ __forceinline__ void wait_vmcnt_le(int n) {
-  switch (n) {
-#define C(k) case k: DSA_WAIT_VMCNT(k); break;
-    C(0) C(1) C(2) C(3) C(4) C(5) C(6) C(7) C(8) C(9) C(10) C(11) C(12) C(13) C(14) C(15) C(16) C(17) C(18) C(19)
-    C(20) C(21) C(22) C(23) C(24) C(25) C(26) C(27) C(28) C(29) C(30) C(31) C(32) C(33) C(34) C(35) C(36) C(37)
-    C(38) C(39) C(40) C(41) C(42) C(43) C(44) C(45) C(46) C(47) C(48)
-#undef C
-    default: DSA_WAIT_VMCNT(0); break;
-  }
-}
-
 // ---------------------------------------------------------------------------------------------
 // pass A: P and dS of every (query, tile)
 // ---------------------------------------------------------------------------------------------
@@ -67,14 +55,13 @@ __device__ __forceinline__ void wait_vmcnt_le(int n) {
 // one key per lane and 16 heads per lane, which is the k-vector layout pass C needs, so P and dS go
 // to HBM as 16-byte chunks without any shuffle.
 template <int STAGES>
-__global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
+__device__ __forceinline__ void pds_body(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
     const __bf16* __restrict__ out, const __bf16* __restrict__ dout, const float* __restrict__ lse,
-    unsigned char* __restrict__ pds, int q0, int cnt, int H, int Skv, int K, int q_start, float sm_scale) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    unsigned char* __restrict__ pds, int q0, int ql, int H, int Skv, int K, int q_start, float sm_scale,
+    unsigned char* smem) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, g = lane >> 5;
-  const int ql = cnt - 1 - (int)blockIdx.x;
   const int qi = q0 + ql;
   const int NT = K / BI;
   int* idx_s = (int*)(smem + STAGES * TILE_BYTES);
@@ -144,7 +131,14 @@ __global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
 
   for (int n = 0; n < ntiles; n++) {
     // operations issued after this tile's gather: 9 per later gather, 4 stores per finished tile
-    wait_vmcnt_le(9 * min(STAGES - 2, ntiles - 1 - n) + 4 * min(n, STAGES - 1));
+    {
+      const int need = 9 * min(STAGES - 2, ntiles - 1 - n) + 4 * min(n, STAGES - 1);
+      constexpr int FULL = 9 * (STAGES - 2) + 4 * (STAGES - 1);
+      if (need >= FULL) { DSA_WAIT_VMCNT(FULL); }                  // steady state
+      else if (need >= 9 * (STAGES - 2)) { DSA_WAIT_VMCNT(9 * (STAGES - 2)); }   // first tiles: fewer stores behind
+      else if (need >= 9) { DSA_WAIT_VMCNT(9); }                   // last tiles: fewer gathers ahead
+      else { DSA_WAIT_VMCNT(0); }
+    }
     __syncthreads();
     if (n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
     const int tile = tlist[n];
@@ -209,16 +203,15 @@ __global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
 // registers nothing filled that gap.  A key-tile operand read from LDS feeds two MFMAs: 112 KB of
 // LDS reads per tile, below the 147 KB the matrix pipe's time allows.
 template <int STAGES>
-__global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
+__device__ __forceinline__ void dq_body(
     const __bf16* __restrict__ kv, const int* __restrict__ ids, const unsigned char* __restrict__ pds,
-    __bf16* __restrict__ dq, int q0, int cnt, int H, int Skv, int K, int q_start, const int* __restrict__ dup_flag) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    __bf16* __restrict__ dq, int q0, int ql, int H, int Skv, int K, int q_start, const int* __restrict__ dup_flag,
+    unsigned char* smem) {
   constexpr int STAGE_BYTES = TILE_BYTES + PDS_KIND_BYTES;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int w = wave & 3, hh = wave >> 2;
   const int r = lane & 31, g = lane >> 5;
-  const int ql = cnt - 1 - (int)blockIdx.x;
   const int qi = q0 + ql;
   const int NT = K / BI;
   int* idx_s = (int*)(smem + STAGES * STAGE_BYTES);
@@ -268,7 +261,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
   // Transfers of a tile: the key rows as nine 128-byte groups per row, thread (key, sub) of either half of
   // the workgroup moving 16 bytes of a group (waves 0-3 take groups 0-4, waves 4-7 groups 5-8), and the
   // 8 KB dS block, 16 bytes per thread.
-  const int per_issue = hh ? 5 : 6;          // transfers per wave and tile
+  // transfers per wave and tile: 6 for waves 0-3, 5 for waves 4-7
   auto issue = [&](int n) {
     const int tile = tlist[n];
     const unsigned sb = lds0 + (unsigned)((n % STAGES) * STAGE_BYTES);
@@ -305,7 +298,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
   };
   for (int n = 0; n < STAGES - 1 && n < ntiles; n++) issue(n);
   for (int n = 0; n < ntiles; n++) {
-    wait_vmcnt_le(per_issue * min(STAGES - 2, ntiles - 1 - n));
+    static_assert(STAGES == 3, "one tile of transfers in flight behind the awaited one");
+    if (n + 1 < ntiles) { if (hh) { DSA_WAIT_VMCNT(5); } else { DSA_WAIT_VMCNT(6); } } else { DSA_WAIT_VMCNT(0); }
     __syncthreads();
     // The two waves of a SIMD (w, 0) and (w, 1) issue their transfers at different times - here and after
     // the second d-tile - so that each does so while the other one feeds the matrix pipe.
@@ -381,32 +375,31 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_kernel(
 // (pass-A layout, read from LDS as stored) also sit in registers, so a column tile is finished by
 // 16 (or 8) back-to-back MFMAs on one accumulator.  Everything else runs in the shadow of the
 // matrix pipe, a few instructions after each MFMA: while column tile c+1 accumulates, tile c is
-// rounded to bf16, transposed through a wave-private LDS strip and stored as 64-byte pieces of
-// its 32 rows at the positions of the key-sorted order; while the last column tile of a tile
-// accumulates, the coefficient registers are refilled for the next tile.  One barrier per tile
-// (the coefficient transfer is shared by the four waves); the per-pair rows are bf16.
-constexpr int DKV_COEF_STAGES = 3;           // coefficient tiles in the LDS ring
-constexpr int DKV_STRIP_STRIDE = 80;         // bytes per row of the wave-private transpose strip
-constexpr int DKV_STRIP_BYTES = BI * DKV_STRIP_STRIDE;
+// rounded to bf16, its four 8-byte pieces per lane are turned into two 16-byte pieces by a trade
+// between the half-waves (the accumulator already holds one key per lane), and these are stored
+// as 32-byte halves of the tile's 64 bytes in each of its 32 rows, at the positions of the
+// key-sorted order; while the last column tile of a tile accumulates, the coefficient registers are
+// refilled for the next tile.  The loop touches LDS for the coefficients only (16 reads per wave
+// and tile).  One barrier per tile (the coefficient transfer is shared by the four waves); the
+// per-pair rows are bf16.
+constexpr int DKV_COEF_STAGES = 5;           // coefficient tiles in the LDS ring
 
 // NC = column tiles of this wave (5 for waves 0 and 1, else 4).
 template <int NC>
 __device__ __forceinline__ void dkv_body(
     const __bf16* __restrict__ q, const __bf16* __restrict__ dout, const int* __restrict__ ids,
     const unsigned char* __restrict__ pds, const int* __restrict__ dst, unsigned char* __restrict__ rows,
-    int q0, int cnt, int H, int Skv, int K, int q_start, int dummy_row, unsigned char* smem) {
+    int q0, int ql, int H, int Skv, int K, int q_start, int dummy_row, unsigned char* smem) {
   constexpr int CST = DKV_COEF_STAGES;
   constexpr int NU = NC == 5 ? 9 : 8;          // units of 8 MFMAs per tile
   // [CST][PDS_TILE_BYTES] coefficient ring, shared with the set-up's per-wave X staging [4][8192] |
-  // [4][DKV_STRIP_BYTES] transpose strips | ids arrays | dst rows of the query [K + 32]
+  // ids arrays | dst rows of the query [K + 32]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, g = lane >> 5;
-  const int ql = cnt - 1 - (int)blockIdx.x;
   const int qi = q0 + ql;
   const int NT = K / BI;
   unsigned char* xs = smem + wave * 8192;
-  unsigned char* strip = smem + CST * PDS_TILE_BYTES + wave * DKV_STRIP_BYTES;
-  int* idx_s = (int*)(smem + CST * PDS_TILE_BYTES + 4 * DKV_STRIP_BYTES);
+  int* idx_s = (int*)(smem + CST * PDS_TILE_BYTES);
   unsigned* tmask = (unsigned*)(idx_s + K);
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
@@ -491,8 +484,12 @@ __device__ __forceinline__ void dkv_body(
   };
   // Vector-memory operations retire in issue order, so "the transfer of tile t has landed" is a
   // bound on the number of operations issued after it: `issued` counts every operation of this
-  // wave, mk_a / mk_b are the counts right after the transfers of the next two tiles.
-  int issued = 0, mk_a = 0, mk_b = 0;
+  // wave, mk[j] is the count right after the transfer of the (j+1)-th tile ahead.  Stores younger
+  // than the awaited transfer stay in flight: the deeper the ring, the more of them.
+  int issued = 0;
+  int mk[CST - 1];
+#pragma unroll
+  for (int j = 0; j < CST - 1; j++) mk[j] = 0;
   auto issue_marked = [&](int n) {
     if (n < ntiles) {
       issue(n);
@@ -504,42 +501,51 @@ __device__ __forceinline__ void dkv_body(
   const unsigned coff = (unsigned)(g * 512 + r * 16);
   bf16x8 cf[16];
   issue_marked(0);
-  mk_a = issue_marked(1);
+  mk[0] = issue_marked(1);
   if (ntiles > 1) { DSA_WAIT_VMCNT(4); } else { DSA_WAIT_VMCNT(0); }
   __syncthreads();
-  mk_b = issue_marked(2);
+#pragma unroll
+  for (int j = 1; j < CST - 1; j++) mk[j] = issue_marked(j + 1);
 #pragma unroll
   for (int k = 0; k < 16; k++) cf[k] = *(const bf16x8*)(smem + k * 1024 + coff);
 
-  // copy-out state: the two 16-byte pieces of the column tile in flight and the row pointers
-  // (row of key it*16 + lane/4, piece lane%4, this wave's first column tile) of the current tile
-  const size_t lane_off = (size_t)(wave * 64 + (lane & 3) * 16);
-  unsigned char* rptr[2];
-  rptr[0] = rptr[1] = rows + (size_t)dummy_row * ROW_BYTES + lane_off;
+  // copy-out state: the rounded column tile in flight (four 8-byte pieces, then two 16-byte ones) and
+  // the pointer to this lane's 16 bytes in the row of its key (lane & 31), first column tile of the wave
+  const size_t lane_off = (size_t)(wave * 64 + g * 16);
+  unsigned char* rptr = rows + (size_t)dummy_row * ROW_BYTES + lane_off;
+  unsigned pc[4][2];
+#pragma unroll
+  for (int j = 0; j < 4; j++) pc[j][0] = pc[j][1] = 0u;
   uint4 piece[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-  const unsigned strip_w = (unsigned)(r * DKV_STRIP_STRIDE + 8 * g);
-  const unsigned strip_r = (unsigned)((lane >> 2) * DKV_STRIP_STRIDE + (lane & 3) * 16);
   f32x16 acc[5];
 #pragma unroll
   for (int e = 0; e < 16; e++) acc[NC - 1][e] = 0.f;   // rounded (to the scratch row) before its first MFMA
 
-  // tasks of column tile ci, spread over MFMA slots: round + transpose-write (4 slots), read back
-  // the two pieces (2 slots), store them (2 slots of the following unit)
+  // tasks of column tile ci, spread over MFMA slots: round (4 slots), trade between the half-waves
+  // (2 slots: piece it = elements 16*it + 8*g .. +7 of the lane's key), store (2 slots of the following unit)
   auto conv = [&](int ci, int j) {
-    uint2 w;
-    w.x = cvt_pk_bf16(acc[ci][4 * j], acc[ci][4 * j + 1]);
-    w.y = cvt_pk_bf16(acc[ci][4 * j + 2], acc[ci][4 * j + 3]);
-    *(uint2*)(strip + strip_w + 16 * j) = w;
+    pc[j][0] = cvt_pk_bf16(acc[ci][4 * j], acc[ci][4 * j + 1]);
+    pc[j][1] = cvt_pk_bf16(acc[ci][4 * j + 2], acc[ci][4 * j + 3]);
   };
-  auto piece_read = [&](int it) { piece[it] = *(const uint4*)(strip + strip_r + it * 16 * DKV_STRIP_STRIDE); };
+  auto piece_read = [&](int it) {
+    const int jj = 2 * it;
+    swap_halves(pc[jj][0], pc[jj + 1][0]);
+    swap_halves(pc[jj][1], pc[jj + 1][1]);
+    piece[it] = make_uint4(pc[jj][0], pc[jj][1], pc[jj + 1][0], pc[jj + 1][1]);
+  };
   auto piece_store = [&](int ci, int it) {
-    *(uint4*)(rptr[it] + ci * 256) = piece[it];
+    *(uint4*)(rptr + ci * 256 + it * 32) = piece[it];
     issued += 1;
   };
+  // Operations a wave has issued, in the steady state, since the transfer it waits for at unit 6 of a
+  // tile (that of the next tile, issued CST - 1 tiles earlier): the stores of unit 7 (and 8) of that
+  // tile, CST - 2 whole tiles of 4 transfers + 2 NC stores, and this tile's stores before unit 6.
+  constexpr int STEADY = 2 + (CST - 2) * (4 + 2 * NC) + (NC == 5 ? 8 : 6);
+  static_assert(STEADY <= 63, "the vector-memory counter holds 63 at most");
 
   for (int n = 0; n < ntiles; n++) {
     const int tile = tlist[n];
-    const int drow0 = dst_s[tile * BI + (lane >> 2)], drow1 = dst_s[tile * BI + 16 + (lane >> 2)];
+    const int drow = dst_s[tile * BI + r];
     const unsigned char* nb = smem + ((n + 1) % CST) * PDS_TILE_BYTES;   // next tile's coefficients
 #pragma unroll
     for (int u = 0; u < NU; u++) {
@@ -550,15 +556,18 @@ __device__ __forceinline__ void dkv_body(
       const int store_ci = p2 == 8 ? 4 : ((p2 & 1) ? p2 >> 1 : -1);
       const bool reload = half == 1 ? u == 7 : u == (NC == 5 ? 8 : 6);
       if (u == 6) {
-        if (n + 1 < ntiles) wait_vmcnt_le(issued - mk_a);
+        // the next tile's coefficients have landed once at most (issued - mk[0]) younger operations
+        // are in flight; anything below the steady-state count (first and last tiles of a query)
+        // waits for everything, which is always enough
+        if (n + 1 < ntiles) {
+          if (issued - mk[0] >= STEADY) { DSA_WAIT_VMCNT(STEADY); } else { DSA_WAIT_VMCNT(0); }
+        }
         __syncthreads();
-        mk_a = mk_b;
-        mk_b = issue_marked(n + CST);
+#pragma unroll
+        for (int j = 0; j + 1 < CST - 1; j++) mk[j] = mk[j + 1];
+        mk[CST - 2] = issue_marked(n + CST);
       }
-      if (u == 2) {                            // all stores of the previous tile are issued
-        rptr[0] = rows + (size_t)drow0 * ROW_BYTES + lane_off;
-        rptr[1] = rows + (size_t)drow1 * ROW_BYTES + lane_off;
-      }
+      if (u == 2) rptr = rows + (size_t)drow * ROW_BYTES + lane_off;      // all stores of the previous tile are issued
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int m = 0; m < 8; m++) {
@@ -592,49 +601,117 @@ __device__ __forceinline__ void dkv_body(
   piece_store(NC - 1, 1);
 }
 
-__global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(
-    const __bf16* __restrict__ q, const __bf16* __restrict__ dout, const int* __restrict__ ids,
-    const unsigned char* __restrict__ pds, const int* __restrict__ dst, unsigned char* __restrict__ rows,
-    int q0, int cnt, int H, int Skv, int K, int q_start, int dummy_row) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  // waves 0 and 1 own five column tiles, waves 2 and 3 four: two copies of the whole body, so that
-  // no branch sits between the MFMAs; every copy meets the same barriers
-  if (threadIdx.x < 128) dkv_body<5>(q, dout, ids, pds, dst, rows, q0, cnt, H, Skv, K, q_start, dummy_row, smem);
-  else dkv_body<4>(q, dout, ids, pds, dst, rows, q0, cnt, H, Skv, K, q_start, dummy_row, smem);
-}
-
 // ---------------------------------------------------------------------------------------------
-// pass D: dKV[key] = sum of the key's rows, ascending query order
+// pass D: dKV[key] = sum of that key's rows, ascending query order
 // ---------------------------------------------------------------------------------------------
-// One 288-thread workgroup per key: 72 column chunks of 8 elements x 4 row groups (row r of the
-// segment goes to group r % 4); the four partial sums are combined in a fixed order, so the result
-// depends only on the segment, never on scheduling.  Pure streaming reads of 1152-byte rows.
-__global__ __launch_bounds__(288) void bwd_reduce_kernel(const unsigned char* __restrict__ rows, const int* __restrict__ start,
-                                                         float* __restrict__ dkv_acc, int Skv, int accumulate) {
-  __shared__ float part[4][DQK];
-  const int key = blockIdx.x;
-  const int ch = threadIdx.x % 72, grp = threadIdx.x / 72;
+// One key per workgroup of 512 threads: 72 column chunks of 8 elements x 7 row groups (row r of the
+// segment goes to group r % 7); the seven partial sums are combined in a fixed order, so the result
+// depends only on the segment, never on scheduling.  Pure streaming reads of 1152-byte rows, RED_FLIGHT
+// of them in flight per thread.
+constexpr int RED_GROUPS = 7;
+constexpr int RED_FLIGHT = 16;               // row pieces a thread has in flight
+__device__ __forceinline__ void reduce_body(const unsigned char* __restrict__ rows, const int* __restrict__ start,
+                                            float* __restrict__ dkv_acc, int key, int accumulate, unsigned char* smem) {
+  float* part = (float*)smem;                  // [RED_GROUPS][DQK]
+  const int tid = threadIdx.x;
+  const int ch = tid % 72, grp = tid / 72;
   const int s0 = start[key], s1 = start[key + 1];
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; e++) acc[e] = 0.f;
-  for (int rr = s0 + grp; rr < s1; rr += 4) {
-    const uint4 v = *(const uint4*)(rows + (size_t)rr * ROW_BYTES + ch * 16);
-    const unsigned w[4] = {v.x, v.y, v.z, v.w};
+  if (grp < RED_GROUPS) {
+    int rr = s0 + grp;
+    for (; rr + (RED_FLIGHT - 1) * RED_GROUPS < s1; rr += RED_FLIGHT * RED_GROUPS) {
+      uint4 v[RED_FLIGHT];
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      acc[2 * e] += __builtin_bit_cast(float, w[e] << 16);
-      acc[2 * e + 1] += __builtin_bit_cast(float, w[e] & 0xffff0000u);
+      for (int u = 0; u < RED_FLIGHT; u++) v[u] = *(const uint4*)(rows + (size_t)(rr + u * RED_GROUPS) * ROW_BYTES + ch * 16);
+#pragma unroll
+      for (int u = 0; u < RED_FLIGHT; u++) {
+        const unsigned w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          acc[2 * e] += __builtin_bit_cast(float, w[e] << 16);
+          acc[2 * e + 1] += __builtin_bit_cast(float, w[e] & 0xffff0000u);
+        }
+      }
     }
-  }
+    for (; rr < s1; rr += RED_GROUPS) {
+      const uint4 v = *(const uint4*)(rows + (size_t)rr * ROW_BYTES + ch * 16);
+      const unsigned w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-  for (int e = 0; e < 8; e++) part[grp][ch * 8 + e] = acc[e];
+      for (int e = 0; e < 4; e++) {
+        acc[2 * e] += __builtin_bit_cast(float, w[e] << 16);
+        acc[2 * e + 1] += __builtin_bit_cast(float, w[e] & 0xffff0000u);
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[grp * DQK + ch * 8 + e] = acc[e];
+  }
   __syncthreads();
-  for (int d = threadIdx.x; d < DQK; d += 288) {
-    const float s = (part[0][d] + part[1][d]) + (part[2][d] + part[3][d]);
+  for (int d = tid; d < DQK; d += 512) {
+    float s = part[d];
+#pragma unroll
+    for (int gq = 1; gq < RED_GROUPS; gq++) s += part[gq * DQK + d];
     float* p = dkv_acc + (size_t)key * DQK + d;
     *p = accumulate ? *p + s : s;
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// kernels: two roles each, chosen per workgroup
+// ---------------------------------------------------------------------------------------------
+// Pass B is bound by LDS reads and leaves HBM nearly idle; pass D is a pure stream of HBM reads and
+// leaves everything else idle; each occupies a whole compute unit (140 KB of LDS, or all its
+// memory-level parallelism).  One launch carries the workgroups of both, alternating in dispatch
+// order, so that at any time about half of the compute units work on either:
+//   bwd_dq_reduce_kernel   pass B of all queries | pass D of all keys      (4.5 ms against 2.6 + 2.75)
+// Workgroup b of a launch with nX and nY workgroups of the two roles: the first 2*min(nX, nY)
+// alternate (even b: X), the rest belong to the longer role.  Within a role, the longest work
+// (latest query, earliest key) comes first.
+// bwd_pds_dkv_kernel can carry pass A of one block of queries beside pass C of another in the same
+// way, but is launched with one role at a time: side by side the two take as long as one after
+// the other (measured with 2 - 64 interleaved blocks), because neither pass gets faster when it has
+// fewer compute units - a compute unit that alternates cold loads (the P / dS tiles) with stores
+// (the rows) drains either queue before it serves the other, which bounds pass C per compute unit
+// at about the rate at which HBM bounds it for the whole chip.
+struct RoleSlot { bool first; int i; };
+__device__ __forceinline__ RoleSlot role_slot(int b, int nX, int nY) {
+  const int n2 = nX < nY ? nX : nY;
+  if (b < 2 * n2) return {(b & 1) == 0, b >> 1};
+  return {nX > nY, n2 + (b - 2 * n2)};
+}
+
+// queries of a role: local query  first + stride * j,  j = 0 .. n-1
+struct QuerySet { int first, stride, n; };
+
+__global__ __launch_bounds__(256, 1) void bwd_pds_dkv_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
+    const __bf16* __restrict__ out, const __bf16* __restrict__ dout, const float* __restrict__ lse,
+    unsigned char* __restrict__ pds, const int* __restrict__ dst, unsigned char* __restrict__ rows,
+    int q0, int H, int Skv, int K, int q_start, float sm_scale, int dummy_row, QuerySet qa, QuerySet qc) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const RoleSlot rs = role_slot((int)blockIdx.x, qa.n, qc.n);
+  if (rs.first) {
+    const int ql = qa.first + qa.stride * (qa.n - 1 - rs.i);
+    pds_body<4>(q, kv, ids, out, dout, lse, pds, q0, ql, H, Skv, K, q_start, sm_scale, smem);
+  } else {
+    const int ql = qc.first + qc.stride * (qc.n - 1 - rs.i);
+    // waves 0 and 1 own five column tiles, waves 2 and 3 four: two copies of the whole body, so that
+    // no branch sits between the MFMAs; every copy meets the same barriers
+    if (threadIdx.x < 128) dkv_body<5>(q, dout, ids, pds, dst, rows, q0, ql, H, Skv, K, q_start, dummy_row, smem);
+    else dkv_body<4>(q, dout, ids, pds, dst, rows, q0, ql, H, Skv, K, q_start, dummy_row, smem);
+  }
+}
+
+__global__ __launch_bounds__(512, 1) void bwd_dq_reduce_kernel(
+    const __bf16* __restrict__ kv, const int* __restrict__ ids, const unsigned char* __restrict__ pds,
+    __bf16* __restrict__ dq, int q0, int cnt, int H, int Skv, int K, int q_start, const int* __restrict__ dup_flag,
+    const unsigned char* __restrict__ rows, const int* __restrict__ start, float* __restrict__ dkv_acc, int n_keys,
+    int accumulate) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const RoleSlot rs = role_slot((int)blockIdx.x, cnt, n_keys);
+  if (rs.first) dq_body<3>(kv, ids, pds, dq, q0, cnt - 1 - rs.i, H, Skv, K, q_start, dup_flag, smem);
+  else reduce_body(rows, start, dkv_acc, rs.i, accumulate, smem);
 }
 
 // fp32 accumulator -> bf16 dKV; NaN everywhere when a query row held a repeated id
@@ -730,17 +807,22 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
 
   const size_t smemA = (size_t)4 * TILE_BYTES + ids_lds_bytes(K) + 16 + 1024;
   const size_t smemB = (size_t)3 * (TILE_BYTES + PDS_KIND_BYTES) + ids_lds_bytes(K);
-  const size_t smemC = (size_t)DKV_COEF_STAGES * PDS_TILE_BYTES + 4 * DKV_STRIP_BYTES + ids_lds_bytes(K) + 16 + (size_t)(K + BI) * 4;
-  if (hipFuncSetAttribute((const void*)bwd_pds_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemA) != hipSuccess ||
-      hipFuncSetAttribute((const void*)bwd_dq_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemB) != hipSuccess ||
-      hipFuncSetAttribute((const void*)bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemC) != hipSuccess)
+  const size_t smemC = (size_t)DKV_COEF_STAGES * PDS_TILE_BYTES + ids_lds_bytes(K) + 16 + (size_t)(K + BI) * 4;
+  const size_t smemAC = smemA > smemC ? smemA : smemC;
+  if (hipFuncSetAttribute((const void*)bwd_pds_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemAC) != hipSuccess ||
+      hipFuncSetAttribute((const void*)bwd_dq_reduce_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemB) != hipSuccess)
     DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_bwd: cannot reserve LDS");
 
-  // optional per-pass timing (profiling entry point only): events between the passes
-  hipEvent_t ev[6];
+  // optional timing (profiling entry point only): events between the launch groups
+  hipEvent_t ev[5];
   if (pass_ms) {
     for (int i = 0; i < 5; i++) pass_ms[i] = 0.f;
-    for (int i = 0; i < 6; i++) if (hipEventCreate(&ev[i]) != hipSuccess) DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_bwd_profile: cannot create events");
+    int made = 0;
+    for (; made < 5; made++) if (hipEventCreate(&ev[made]) != hipSuccess) break;
+    if (made < 5) {
+      for (int i = 0; i < made; i++) hipEventDestroy(ev[i]);
+      DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_bwd_profile: cannot create events");
+    }
   }
 #define DSA_MARK(i) do { if (pass_ms) hipEventRecord(ev[i], st); } while (0)
   bool first = true;
@@ -758,23 +840,24 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
     const int* sids = sort_ids ? sorted : ids + (size_t)q0 * K;      // row ql belongs to query q0 + ql
     DSA_MARK(1);
-    bwd_pds_kernel<4><<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out,
-                                                          (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);
-    DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(P, dS)");
-    DSA_MARK(2);
-    bwd_dq_kernel<3><<<dim3(cnt), dim3(512), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv, K, q_start, dup_flag);
-    DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ)");
+    // Pass A, then pass C (the same kernel with one role each: see the note at the kernel).
+    const QuerySet all = {0, 1, cnt}, none = {0, 1, 0};
+    for (int c = 0; c < 2; c++) {
+      bwd_pds_dkv_kernel<<<dim3(cnt), dim3(256), smemAC, st>>>(
+          (const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out, (const __bf16*)dout, lse, pds, dstp, rows, q0, H,
+          Skv, K, q_start, sm_scale, p.chunk * K, c == 0 ? all : none, c == 0 ? none : all);
+      DSA_CHECK_LAUNCH(c == 0 ? "dsa_sparse_mla_bwd(P, dS)" : "dsa_sparse_mla_bwd(dKV rows)");
+      if (c == 0) DSA_MARK(2);
+    }
     DSA_MARK(3);
-    bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, sids, pds, dstp, rows, q0, cnt,
-                                                       H, Skv, K, q_start, p.chunk * K);
-    DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV rows)");
+    // Pass B of every query beside pass D of every key.
+    bwd_dq_reduce_kernel<<<dim3(cnt + Skv), dim3(512), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv,
+                                                                   K, q_start, dup_flag, rows, start, acc, Skv, first ? 0 : 1);
+    DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ | dKV reduce)");
     DSA_MARK(4);
-    bwd_reduce_kernel<<<dim3(Skv), dim3(288), 0, st>>>(rows, start, acc, Skv, first ? 0 : 1);
-    DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV reduce)");
-    DSA_MARK(5);
     if (pass_ms) {
-      hipEventSynchronize(ev[5]);
-      for (int i = 0; i < 5; i++) { float ms = 0.f; hipEventElapsedTime(&ms, ev[i], ev[i + 1]); pass_ms[i] += ms; }
+      hipEventSynchronize(ev[4]);
+      for (int i = 0; i < 4; i++) { float ms = 0.f; hipEventElapsedTime(&ms, ev[i], ev[i + 1]); pass_ms[i] += ms; }
     }
     first = false;
   }
@@ -784,7 +867,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   cast_bf16_kernel<<<dim3(2048), dim3(256), 0, st>>>(acc, (unsigned short*)dkv, (size_t)Skv * DQK, dup_flag);
   DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(cast)");
   (void)NT;
-  if (pass_ms) for (int i = 0; i < 6; i++) hipEventDestroy(ev[i]);
+  if (pass_ms) for (int i = 0; i < 5; i++) hipEventDestroy(ev[i]);
 #undef DSA_MARK
   return DSA_OK;
 }
