@@ -9,7 +9,8 @@ One step = one pass of the hot path at sequence length 8192 with all inputs resi
 Prints ONE JSON line.  `value` is the sparse-MLA forward+backward rate in TFLOP/s (algorithmic
 flops: 2*H*(576+512) forward and 2*H*(3*576+2*512) backward per valid (query, key) pair, pairs =
 sum_q min(prefix_q, 2048)); the indexer + top-k rate in tokens/s is reported next to it.
-`roofline` describes the longest-running kernel of the step, timed live with HIP events;
+`roofline` describes the longest-running launch of the step, timed live with HIP events, against
+the bf16 MFMA peak (its share of the algorithmic flops); the HBM bytes the design moves are beside it;
 `cpu_baseline` is the CPU oracle (a PyTorch restatement of the reference's math) on a bounded
 sample of the same workload, on this box's host cores.
 """
@@ -61,6 +62,20 @@ def cpu_baseline(inp, iq, ik, w, n_queries=2048):
     }
 
 
+def kernel_sources_sha256():
+    """Digest of the kernel sources: a committed counter profile counts only for the sources it was taken with."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha256()
+    base = os.path.join(ROOT, "loongforge_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(base, "*.hip")) + glob.glob(os.path.join(base, "*.h"))):
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -83,6 +98,7 @@ def main():
         print("bench.py needs a HIP device", file=sys.stderr)
         sys.exit(1)
     lib = _lib.load()
+    blib = _lib.load_bench()         # measurement aids: the backward with per-launch timing, plain movers, an MFMA loop
     dev = torch.device("cuda:0")
 
     # ---- synthetic inputs (CPU RNG, then resident in HBM) ------------------------------------
@@ -118,7 +134,7 @@ def main():
         return torch.cuda.Event(enable_timing=True)
 
     t_idx = t_fwd = t_bwd = 0.0
-    t_pass = [0.0] * 5
+    t_pass = [0.0] * 5           # launch groups of the backward: order, pass A, pass C, passes B | D
     t_logits = t_topk = 0.0
     wall = 0.0
     for step in range(args.warmup + args.steps):
@@ -141,10 +157,10 @@ def main():
         _lib.check(lib.dsa_sparse_mla_fwd(q.data_ptr(), kv.data_ptr(), idx.data_ptr(), S, H, S, K, 0, inp.sm_scale, DV,
                                           out.data_ptr(), lse.data_ptr(), None, 0, stream), "fwd")
         e[3].record()
-        _lib.check(lib.dsa_sparse_mla_bwd_profile(q.data_ptr(), kv.data_ptr(), out.data_ptr(), do.data_ptr(),
-                                                  idx.data_ptr(), lse.data_ptr(), S, H, S, K, 0, inp.sm_scale, DV,
-                                                  dq.data_ptr(), dkv.data_ptr(), ws.data_ptr(), wsb, stream, pass_ms),
-                   "bwd")
+        _lib.check(blib.dsa_sparse_mla_bwd_profile(q.data_ptr(), kv.data_ptr(), out.data_ptr(), do.data_ptr(),
+                                                   idx.data_ptr(), lse.data_ptr(), S, H, S, K, 0, inp.sm_scale, DV,
+                                                   dq.data_ptr(), dkv.data_ptr(), ws.data_ptr(), wsb, stream, pass_ms),
+                   "bwd", blib)
         e[4].record()
         torch.cuda.synchronize()
         if timed:
@@ -186,6 +202,8 @@ def main():
     _, _, p_raw = ops.sparse_mla_fwd(q, kv, idx, 0, inp.sm_scale, DV, True)
     t_dist, _ = timed(lambda: ops.attn_dist(p_raw, inp.sm_scale))
     del p_raw, g_sel
+    # the same distribution without the [S, H, K] logits: recomputed from q, kv and lse
+    t_dist_qk, _ = timed(lambda: ops.attn_dist_qk(q, kv, idx, lse, 0, inp.sm_scale, H))
     # one forward with cold caches (a 1 GiB fill evicts L2 and the memory-side cache first)
     flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     flush.fill_(1)
@@ -227,10 +245,10 @@ def main():
     if row_bytes + src_bytes + 256 <= wsb:
         src_ptr = ws.data_ptr() + (row_bytes + 255) // 256 * 256
         sink = torch.zeros(16, dtype=torch.uint8, device=dev)
-        t_rows, _ = timed(lambda: _lib.check(lib.dsa_probe_hbm_rows(src_ptr, ws.data_ptr(), S, rows_per_wg, 3, 1, stream),
-                                             "probe rows"))
-        t_read, _ = timed(lambda: _lib.check(lib.dsa_probe_hbm_read(ws.data_ptr(), row_bytes, sink.data_ptr(), stream),
-                                             "probe read"))
+        t_rows, _ = timed(lambda: _lib.check(blib.dsa_probe_hbm_rows(src_ptr, ws.data_ptr(), S, rows_per_wg, 3, 1, stream),
+                                             "probe rows", blib))
+        t_read, _ = timed(lambda: _lib.check(blib.dsa_probe_hbm_read(ws.data_ptr(), row_bytes, sink.data_ptr(), stream),
+                                             "probe read", blib))
         mover = {"rows_written_scattered_plus_stream_read_gbps": round((row_bytes + src_bytes) / (t_rows * 1e-3) / 1e9, 1),
                  "stream_read_gbps": round(row_bytes / (t_read * 1e-3) / 1e9, 1),
                  "note": "plain movers with the byte counts and access shape of bwd_dkv_kernel and bwd_reduce_kernel"}
@@ -238,46 +256,54 @@ def main():
     # what the matrix pipes sustain when a kernel issues nothing but bf16 MFMAs (about 20 ms of them)
     probe_flops = ctypes.c_double(0.0)
     sink4 = torch.zeros(4, dtype=torch.float32, device=dev)
-    t_mfma, _ = timed(lambda: _lib.check(lib.dsa_probe_mfma_bf16(2048, 10000, sink4.data_ptr(), ctypes.byref(probe_flops),
-                                                                 stream), "probe mfma"))
+    t_mfma, _ = timed(lambda: _lib.check(blib.dsa_probe_mfma_bf16(2048, 10000, sink4.data_ptr(), ctypes.byref(probe_flops),
+                                                                  stream), "probe mfma", blib))
     mfma_sustained = probe_flops.value / (t_mfma * 1e-3) / 1e12
 
     mla_tflops = (flops_fwd + flops_bwd) / ((t_fwd + t_bwd) * 1e-3) / 1e12
-    # ---- roofline of the longest-running kernel of the step ---------------------------------------
-    # Per kernel: algorithmic flops and algorithmic HBM bytes of one launch.  Gathered key rows are
-    # not counted as HBM bytes (the 9.4 MB latent buffer stays in cache); the bound is the roofline
-    # that gives the longer minimum time.
+    # ---- roofline of the longest-running launch of the step ----------------------------------------
+    # Every sparse-MLA kernel is priced against the bf16 MFMA peak with its share of the algorithmic
+    # flops (2*H*d per (query, key) pair and product).  Next to it: the HBM bytes this build's
+    # design moves in that launch (its intermediates included), the bytes an ideal backward would
+    # move, and - when a counter profile of exactly these sources is committed - the measured traffic.
     nq = float(S)
     b_q, b_do, b_o = nq * H * DQK * 2, nq * H * DV * 2, nq * H * DV * 2
     b_pds = 512.0 * pairs                     # bf16 P and dS, 128 heads, per pair
     b_rows = 1152.0 * pairs                   # one bf16 row of 576 per pair
-    pass_names = ["order", "bwd_pds_kernel (S, dP -> P, dS)", "bwd_dq_kernel (dQ)", "bwd_dkv_kernel (dKV rows)",
-                  "bwd_reduce_kernel (ordered dKV sum)"]
-    pass_flops = [0.0, 2.0 * H * (DQK + DV) * pairs, 2.0 * H * DQK * pairs, 2.0 * H * (DQK + DV) * pairs, 0.0]
-    pass_bytes = [8.0 * pairs, b_q + b_do + b_o + b_pds, 0.5 * b_pds + b_q, b_pds + b_rows + b_q + b_do,
-                  b_rows + S * DQK * 4.0]
+    b_dq, b_dkv = nq * H * DQK * 2, float(S) * DQK * 2
+    pass_names = ["order", "bwd_pds_kernel (S, dP -> P, dS)", "bwd_dkv_kernel (dKV rows)",
+                  "bwd_dq_reduce_kernel (dQ beside the ordered dKV sum)"]
+    pass_flops = [0.0, 2.0 * H * (DQK + DV) * pairs, 2.0 * H * (DQK + DV) * pairs, 2.0 * H * DQK * pairs]
+    pass_bytes = [8.0 * pairs, b_q + b_do + b_o + b_pds, b_pds + b_rows + b_q + b_do,
+                  0.5 * b_pds + b_dq + b_rows + S * DQK * 4.0]
     kernels = [("mla_fwd_kernel", t_fwd, flops_fwd, b_q + b_o)]
-    kernels += [(pass_names[i], t_pass[i], pass_flops[i], pass_bytes[i]) for i in range(5)]
+    kernels += [(pass_names[i], t_pass[i], pass_flops[i], pass_bytes[i]) for i in range(4)]
     name, t_dom, f_dom, b_dom = max(kernels, key=lambda k: k[1])
-    traffic = None
+    traffic, traffic_note = None, "no counter profile committed for these kernel sources"
     tpath = os.path.join(ROOT, "profiles", "traffic.json")   # HBM bytes per launch from rocprofv3 counter runs
     if os.path.exists(tpath):
         with open(tpath) as fh:
-            traffic = json.load(fh).get(name.split(" ")[0], {}).get("hbm_bytes_per_launch")
-    if f_dom / (PEAK_BF16 * 1e12) >= b_dom / 8e12:
-        roofline = {"kernel": name, "bound": "mfma", "achieved": round(f_dom / (t_dom * 1e-3) / 1e12, 1),
-                    "peak": PEAK_BF16, "unit": "TFLOP/s", "traffic": traffic}
-    else:
-        roofline = {"kernel": name, "bound": "hbm", "achieved": round(b_dom / (t_dom * 1e-3) / 1e9, 1), "peak": 8000.0,
-                    "unit": "GB/s", "traffic": traffic}
+            tj = json.load(fh)
+        if tj.get("sources_sha256") == kernel_sources_sha256():
+            traffic = tj.get("kernels", {}).get(name.split(" ")[0], {}).get("hbm_bytes_per_launch")
+            traffic_note = "rocprofv3 FETCH_SIZE + WRITE_SIZE of profiles/traffic.json, taken with these kernel sources"
+        else:
+            traffic_note = "profiles/traffic.json was taken with other kernel sources: dropped"
+    roofline = {"kernel": name, "bound": "mfma", "achieved": round(f_dom / (t_dom * 1e-3) / 1e12, 1),
+                "peak": PEAK_BF16, "unit": "TFLOP/s", "traffic": traffic, "traffic_note": traffic_note}
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
     roofline["avg_launch_ms"] = round(t_dom, 3)
-    roofline["algorithmic_bytes"] = b_dom
     roofline["algorithmic_flops"] = f_dom
-    if mover is not None and roofline["bound"] == "hbm":
-        # the same launch against the measured rate of a plain mover of its traffic shape
-        ref = mover["rows_written_scattered_plus_stream_read_gbps" if name.startswith("bwd_dkv") else "stream_read_gbps"]
-        roofline["frac_of_plain_mover"] = round(roofline["achieved"] / ref, 4)
+    roofline["design_hbm_bytes"] = b_dom          # what this build's passes move in that launch, intermediates included
+    roofline["design_hbm_gbps"] = round(b_dom / (t_dom * 1e-3) / 1e9, 1)
+    roofline["design_hbm_frac_of_8tbps"] = round(b_dom / (t_dom * 1e-3) / 8e12, 4)
+    # the whole backward: bytes an ideal implementation moves (Q, dO, O in; dQ, dKV out) against this design's
+    ideal_bwd = b_q + b_do + b_o + b_dq + b_dkv
+    design_bwd = sum(pass_bytes)
+    roofline["backward_hbm_bytes"] = {"ideal": ideal_bwd, "design": design_bwd, "ratio": round(design_bwd / ideal_bwd, 2)}
+    roofline["path_frac_of_bf16_mfma_peak"] = round(mla_tflops / PEAK_BF16, 4)
+    if mover is not None:
+        roofline["plain_mover_gbps"] = mover
     if args.copy_calibration:
         # a plain 1 GiB device copy: the known-size kernel the HBM counters are scaled by
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -305,7 +331,7 @@ def main():
         "mla_fwd_ms": round(t_fwd, 3), "mla_bwd_ms": round(t_bwd, 3),
         "mla_fwd_tflops": round(flops_fwd / (t_fwd * 1e-3) / 1e12, 1),
         "mla_bwd_tflops": round(flops_bwd / (t_bwd * 1e-3) / 1e12, 1),
-        "mla_bwd_pass_ms": {pass_names[i]: round(t_pass[i], 3) for i in range(5)},
+        "mla_bwd_pass_ms": {pass_names[i]: round(t_pass[i], 3) for i in range(4)},
         "indexer_topk_ms": round(t_idx, 3),
         "indexer_topk_tokens_per_s": round(S / (t_idx * 1e-3), 1),
         "indexer_topk_fp8_tflops": round(flops_idx / (t_idx * 1e-3) / 1e12, 1),
@@ -315,6 +341,7 @@ def main():
         "indexer_bwd_ms": round(t_ibwd, 3),
         "attn_dist_ms": round(t_dist, 3),
         "attn_dist_gbps": round((2.0 * S * H * K + 4.0 * S * K) / (t_dist * 1e-3) / 1e9, 1),
+        "attn_dist_from_q_kv_lse_ms": round(t_dist_qk, 3),
         "mla_fwd_ms_cold_caches": round(t_fwd_cold, 3),
         "mla_fwd_gather_gbps": round(2.0 * DQK * pairs / (t_fwd * 1e-3) / 1e9, 1),
         "nominal": {"note": "the same times priced on S*K pairs and S*S logits, as the reference's own print-outs do",

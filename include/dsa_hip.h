@@ -188,19 +188,6 @@ int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out, const voi
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Profiling variant of dsa_sparse_mla_bwd: same arguments and results, plus the time of each pass
- * in milliseconds, measured with HIP events on `stream` and summed over query chunks:
- *   pass_ms[0] key-sorted order   [1] P and dS   [2] dQ   [3] per-pair dKV rows   [4] ordered dKV reduce
- * It creates and destroys HIP events and waits for the stream before returning, so it is for
- * benchmarks only.  No counterpart in the reference (its kernels are timed with do_bench from
- * Python, ops/tilelang_ops/sparse_mla_bwd.py:359-368).
- */
-int dsa_sparse_mla_bwd_profile(const void* q, const void* kv, const void* out, const void* dout,
-                               const int32_t* ids, const float* lse, int S, int H, int Skv, int K,
-                               int q_start, float sm_scale, int d_v, void* dq, void* dkv,
-                               void* workspace, size_t workspace_bytes, void* stream, float* pass_ms);
-
-/*
  * Head-averaged attention distribution over the selected slots:
  *   target[i,t] = (1/H) sum_h softmax_t(p_out[i,h,:] * sm_scale)[t]
  * Replaces triton_attn_dist, dsa_fused_kernels.py:1844-1955.  `ld_s` / `ld_h` are the element
@@ -209,6 +196,21 @@ int dsa_sparse_mla_bwd_profile(const void* q, const void* kv, const void* out, c
  */
 int dsa_attn_dist(const void* p_out, int p_out_f32, int S, int H, int K, int64_t ld_s,
                   int64_t ld_h, float sm_scale, float* target, void* stream);
+
+/*
+ * The same distribution without materialised logits: recomputed from q, kv, ids and the forward's
+ * natural-log lse,
+ *   target[i,t] = (1/heads_in_mean) sum_{h < heads_in_mean} exp(q[i,h,:] . kv[ids[i,t],:] * sm_scale - lse[i,h])
+ * (0 for invalid slots; validity as in dsa_sparse_mla_fwd), which is mean_h softmax_t when lse[i,h]
+ * is the log-sum-exp over the same slots.  Replaces the pair `return_p_out=True` +
+ * triton_attn_dist of the training path (loongforge/models/common/experimental_attention_variant/
+ * dsa_fused.py:903-929): the [S, H, K] logits (4.3 GB at seq 8192) are neither written nor read.
+ * heads_in_mean < H leaves out padded heads, as the slice at dsa_fused.py:915-917 does.
+ *   q [S, H, 576] bf16   kv [Skv, 576] bf16   ids [S, K] i32 (K % 64 == 0, K <= 4096)   lse [S, H] f32
+ */
+int dsa_attn_dist_qk(const void* q, const void* kv, const int32_t* ids, const float* lse, int S, int H,
+                     int heads_in_mean, int Skv, int K, int q_start, float sm_scale, float* target,
+                     void* stream);
 
 /*
  * Rotary position embedding of the MLA query / key rows, fused with the copies around it.  Per
@@ -251,26 +253,6 @@ int dsa_rope_headsum_inverse(const void* grad, int64_t g_tok, int64_t g_head, vo
                              int emb_dim, const void* cos, const void* sin, int cos_sin_f32,
                              const int32_t* positions, int batch, int tokens, int heads, int in_pairing,
                              void* stream);
-
-/*
- * Measurement aids; no counterpart in the reference.  Plain data movers with the traffic shape of
- * the two bandwidth-bound backward passes, and a kernel of nothing but bf16 MFMAs, so that a
- * benchmark can quote the kernels against what the memory system and the matrix pipes give a
- * kernel that does nothing else.
- *
- * dsa_probe_hbm_rows: `workgroups` x `rows_per_workgroup` (a multiple of 4) rows of 1152 bytes are
- * written to `rows` (at permuted row positions when scatter != 0, in order otherwise) while each
- * workgroup streams 4608 bytes from `src` on read_fifths (0..5) of every 5 steps of 4 rows; with
- * n = rows_per_workgroup / 4 steps, src must hold
- * workgroups * (n / 5 * read_fifths + min(n % 5, read_fifths)) * 4608 bytes.
- * dsa_probe_hbm_read: streams `bytes` from src; sink16 points at 16 writable bytes.
- */
-int dsa_probe_hbm_rows(const void* src, void* rows, int workgroups, int rows_per_workgroup, int read_fifths,
-                       int scatter, void* stream);
-int dsa_probe_hbm_read(const void* src, size_t bytes, void* sink16, void* stream);
-/* dsa_probe_mfma_bf16: `workgroups` x 4 waves each issue iters x 16 v_mfma_f32_32x32x16_bf16 and nothing else;
- * *flops (may be NULL) receives the flop count of the launch; sink4 points at 4 writable bytes. */
-int dsa_probe_mfma_bf16(int workgroups, int iters, void* sink4, double* flops, void* stream);
 
 #ifdef __cplusplus
 }

@@ -30,12 +30,19 @@ SIGNATURES = {
     "dsa_sparse_mla_fwd_ex": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _i, _vp, _i, _vp]),
     "dsa_sparse_mla_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "dsa_sparse_mla_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _sz, _vp]),
-    "dsa_sparse_mla_bwd_profile": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _sz, _vp,
-                                        _vp]),
     "dsa_attn_dist": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _f, _vp, _vp]),
+    "dsa_attn_dist_qk": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "dsa_rope_rows": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _i, _vp, _i64, _i64, _vp, _i64, _i64, _i, _vp, _vp, _i, _vp,
                            _i, _i, _i, _i, _i, _i, _vp]),
     "dsa_rope_headsum_inverse": (_i, [_vp, _i64, _i64, _vp, _i64, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
+}
+
+# libdsa_bench.so: measurement aids for the benchmark (include/dsa_hip_bench.h), not part of the boundary
+BENCH_LIB_PATH = os.path.join(_HERE, "libdsa_bench.so")
+BENCH_SIGNATURES = {
+    "dsa_last_error": (_c.c_char_p, []),
+    "dsa_sparse_mla_bwd_profile": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _sz, _vp,
+                                        _vp]),
     "dsa_probe_hbm_rows": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "dsa_probe_hbm_read": (_i, [_vp, _sz, _vp, _vp]),
     "dsa_probe_mfma_bf16": (_i, [_i, _i, _vp, _vp, _vp]),
@@ -68,10 +75,24 @@ def load():
         return _lib
 
 
-def check(rc, what):
-    """Turns a negative status into an exception carrying dsa_last_error()."""
+def load_bench():
+    """The benchmark-only library (its own copy of the backward with per-launch timing, and plain
+    data movers / MFMA loops to quote the kernels against)."""
+    if not os.path.exists(BENCH_LIB_PATH):
+        raise DsaError("libdsa_bench.so is missing at %s; build it with `python -m loongforge_amd.csrc.build`"
+                       % BENCH_LIB_PATH)
+    lib = ctypes.CDLL(BENCH_LIB_PATH)
+    for name, (res, args) in BENCH_SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+def check(rc, what, lib=None):
+    """Turns a negative status into an exception carrying dsa_last_error() (of `lib`, default the kernels')."""
     if rc != 0:
-        msg = load().dsa_last_error().decode("utf-8", "replace")
+        msg = (lib or load()).dsa_last_error().decode("utf-8", "replace")
         if rc == -1:
             raise ValueError("%s: %s" % (what, msg))
         raise DsaError("%s failed (status %d): %s" % (what, rc, msg))

@@ -3,7 +3,8 @@
 // same bytes the same way: 1152-byte rows written at scattered row positions beside a streaming read
 // (the dKV-row pass), and a pure streaming read (the ordered dKV sum).  The benchmark quotes the
 // passes against these rates next to the nominal HBM peak.
-#include "dsa_common.h"
+#include "../dsa_common.h"
+#include "../../../include/dsa_hip_bench.h"
 
 namespace {
 

@@ -21,9 +21,7 @@ namespace {
 constexpr int D = 128;          // indexer head dim (bytes per fp8 row)
 constexpr int BK = 128;         // keys per LDS tile
 constexpr int TILE_BYTES = BK * D;
-#ifndef IDX_QW
-#define IDX_QW 1                // queries per wave
-#endif
+constexpr int IDX_QW = 1;       // queries per wave (one: 122 registers, four waves per SIMD)
 constexpr int QB = 8;           // queries per workgroup
 
 __device__ __forceinline__ int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }

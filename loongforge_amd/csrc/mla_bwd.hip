@@ -27,26 +27,6 @@ constexpr int PDS_KIND_BYTES = 8192;
 constexpr int ROW_BYTES = DQK * 2;           // one pair row of the dKV buffer
 
 // ---------------------------------------------------------------------------------------------
-// MFMA through inline asm with explicit register files ("v" architectural, "a" accumulation).
-// Back-to-back MFMAs accumulating into the same registers need no software wait states; whoever
-// reads a finished accumulator with a non-MFMA instruction calls mfma_done first.
-// ---------------------------------------------------------------------------------------------
-#define DSA_MFMA_FN(name, ACC, A, B)                                                              \
-  __device__ __forceinline__ void name##_first(f32x16& acc, const bf16x8& a, const bf16x8& b) {   \
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&" ACC(acc) : A(a), B(b));           \
-  }                                                                                               \
-  __device__ __forceinline__ void name(f32x16& acc, const bf16x8& a, const bf16x8& b) {           \
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+" ACC(acc) : A(a), B(b));           \
-  }
-DSA_MFMA_FN(mfma_v_av, "v", "a", "v")   // acc VGPR, A in AGPR, B in VGPR
-DSA_MFMA_FN(mfma_v_vv, "v", "v", "v")
-DSA_MFMA_FN(mfma_a_vv, "a", "v", "v")
-DSA_MFMA_FN(mfma_a_av, "a", "a", "v")
-#undef DSA_MFMA_FN
-__device__ __forceinline__ void mfma_done_v(f32x16& acc) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(acc)); }
-__device__ __forceinline__ void mfma_done_a(f32x16& acc) { asm volatile("s_nop 15\n\ts_nop 3" : "+a"(acc)); }
-
-// ---------------------------------------------------------------------------------------------
 // pass A: P and dS of every (query, tile)
 // ---------------------------------------------------------------------------------------------
 // One workgroup per query, wave w owns heads [32w, 32w+32).  S = Q.KV^T and dP = dO.V^T share the
@@ -668,12 +648,12 @@ __device__ __forceinline__ void reduce_body(const unsigned char* __restrict__ ro
 // Workgroup b of a launch with nX and nY workgroups of the two roles: the first 2*min(nX, nY)
 // alternate (even b: X), the rest belong to the longer role.  Within a role, the longest work
 // (latest query, earliest key) comes first.
-// bwd_pds_dkv_kernel can carry pass A of one block of queries beside pass C of another in the same
-// way, but is launched with one role at a time: side by side the two take as long as one after
-// the other (measured with 2 - 64 interleaved blocks), because neither pass gets faster when it has
-// fewer compute units - a compute unit that alternates cold loads (the P / dS tiles) with stores
-// (the rows) drains either queue before it serves the other, which bounds pass C per compute unit
-// at about the rate at which HBM bounds it for the whole chip.
+// Passes A and C, carried by one launch in the same way (pass A of one block of queries beside
+// pass C of the block before it, 2 - 64 interleaved blocks), took as long side by side as one after
+// the other: neither gets faster when it has fewer compute units - a compute unit that alternates
+// cold loads (the P / dS tiles) with stores (the rows) drains either queue before it serves the
+// other, which bounds pass C per compute unit at about the rate at which HBM bounds it for the
+// whole chip.  They are separate kernels.
 struct RoleSlot { bool first; int i; };
 __device__ __forceinline__ RoleSlot role_slot(int b, int nX, int nY) {
   const int n2 = nX < nY ? nX : nY;
@@ -681,26 +661,24 @@ __device__ __forceinline__ RoleSlot role_slot(int b, int nX, int nY) {
   return {nX > nY, n2 + (b - 2 * n2)};
 }
 
-// queries of a role: local query  first + stride * j,  j = 0 .. n-1
-struct QuerySet { int first, stride, n; };
-
-__global__ __launch_bounds__(256, 1) void bwd_pds_dkv_kernel(
+__global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
     const __bf16* __restrict__ out, const __bf16* __restrict__ dout, const float* __restrict__ lse,
-    unsigned char* __restrict__ pds, const int* __restrict__ dst, unsigned char* __restrict__ rows,
-    int q0, int H, int Skv, int K, int q_start, float sm_scale, int dummy_row, QuerySet qa, QuerySet qc) {
+    unsigned char* __restrict__ pds, int q0, int cnt, int H, int Skv, int K, int q_start, float sm_scale) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  const RoleSlot rs = role_slot((int)blockIdx.x, qa.n, qc.n);
-  if (rs.first) {
-    const int ql = qa.first + qa.stride * (qa.n - 1 - rs.i);
-    pds_body<4>(q, kv, ids, out, dout, lse, pds, q0, ql, H, Skv, K, q_start, sm_scale, smem);
-  } else {
-    const int ql = qc.first + qc.stride * (qc.n - 1 - rs.i);
-    // waves 0 and 1 own five column tiles, waves 2 and 3 four: two copies of the whole body, so that
-    // no branch sits between the MFMAs; every copy meets the same barriers
-    if (threadIdx.x < 128) dkv_body<5>(q, dout, ids, pds, dst, rows, q0, ql, H, Skv, K, q_start, dummy_row, smem);
-    else dkv_body<4>(q, dout, ids, pds, dst, rows, q0, ql, H, Skv, K, q_start, dummy_row, smem);
-  }
+  pds_body<4>(q, kv, ids, out, dout, lse, pds, q0, cnt - 1 - (int)blockIdx.x, H, Skv, K, q_start, sm_scale, smem);
+}
+
+__global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ dout, const int* __restrict__ ids,
+    const unsigned char* __restrict__ pds, const int* __restrict__ dst, unsigned char* __restrict__ rows,
+    int q0, int cnt, int H, int Skv, int K, int q_start, int dummy_row) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int ql = cnt - 1 - (int)blockIdx.x;
+  // waves 0 and 1 own five column tiles, waves 2 and 3 four: two copies of the whole body, so that
+  // no branch sits between the MFMAs; every copy meets the same barriers
+  if (threadIdx.x < 128) dkv_body<5>(q, dout, ids, pds, dst, rows, q0, ql, H, Skv, K, q_start, dummy_row, smem);
+  else dkv_body<4>(q, dout, ids, pds, dst, rows, q0, ql, H, Skv, K, q_start, dummy_row, smem);
 }
 
 __global__ __launch_bounds__(512, 1) void bwd_dq_reduce_kernel(
@@ -808,8 +786,8 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   const size_t smemA = (size_t)4 * TILE_BYTES + ids_lds_bytes(K) + 16 + 1024;
   const size_t smemB = (size_t)3 * (TILE_BYTES + PDS_KIND_BYTES) + ids_lds_bytes(K);
   const size_t smemC = (size_t)DKV_COEF_STAGES * PDS_TILE_BYTES + ids_lds_bytes(K) + 16 + (size_t)(K + BI) * 4;
-  const size_t smemAC = smemA > smemC ? smemA : smemC;
-  if (hipFuncSetAttribute((const void*)bwd_pds_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemAC) != hipSuccess ||
+  if (hipFuncSetAttribute((const void*)bwd_pds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemA) != hipSuccess ||
+      hipFuncSetAttribute((const void*)bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemC) != hipSuccess ||
       hipFuncSetAttribute((const void*)bwd_dq_reduce_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemB) != hipSuccess)
     DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_bwd: cannot reserve LDS");
 
@@ -840,15 +818,13 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
     const int* sids = sort_ids ? sorted : ids + (size_t)q0 * K;      // row ql belongs to query q0 + ql
     DSA_MARK(1);
-    // Pass A, then pass C (the same kernel with one role each: see the note at the kernel).
-    const QuerySet all = {0, 1, cnt}, none = {0, 1, 0};
-    for (int c = 0; c < 2; c++) {
-      bwd_pds_dkv_kernel<<<dim3(cnt), dim3(256), smemAC, st>>>(
-          (const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out, (const __bf16*)dout, lse, pds, dstp, rows, q0, H,
-          Skv, K, q_start, sm_scale, p.chunk * K, c == 0 ? all : none, c == 0 ? none : all);
-      DSA_CHECK_LAUNCH(c == 0 ? "dsa_sparse_mla_bwd(P, dS)" : "dsa_sparse_mla_bwd(dKV rows)");
-      if (c == 0) DSA_MARK(2);
-    }
+    bwd_pds_kernel<<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out,
+                                                       (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);
+    DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(P, dS)");
+    DSA_MARK(2);
+    bwd_dkv_kernel<<<dim3(cnt), dim3(256), smemC, st>>>((const __bf16*)q, (const __bf16*)dout, sids, pds, dstp, rows, q0, cnt,
+                                                       H, Skv, K, q_start, p.chunk * K);
+    DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV rows)");
     DSA_MARK(3);
     // Pass B of every query beside pass D of every key.
     bwd_dq_reduce_kernel<<<dim3(cnt + Skv), dim3(512), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv,
@@ -879,6 +855,7 @@ extern "C" int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out
                   stream, nullptr);
 }
 
+#ifdef DSA_BENCH_BUILD     // the benchmark library compiles this file a second time, with the timed entry point
 extern "C" int dsa_sparse_mla_bwd_profile(const void* q, const void* kv, const void* out, const void* dout,
                                           const int32_t* ids, const float* lse, int S, int H, int Skv, int K, int q_start,
                                           float sm_scale, int d_v, void* dq, void* dkv, void* workspace,
@@ -887,3 +864,4 @@ extern "C" int dsa_sparse_mla_bwd_profile(const void* q, const void* kv, const v
   return bwd_impl(q, kv, out, dout, ids, lse, S, H, Skv, K, q_start, sm_scale, d_v, dq, dkv, workspace, workspace_bytes,
                   stream, pass_ms);
 }
+#endif

@@ -13,31 +13,12 @@
 // one cross-lane exchange per tile; the accumulator layout of S^T is, up to a fixed permutation
 // of the keys inside a tile, the B-operand layout of the second product, so P never touches LDS.
 // MFMA-bound: 2*H*(576+512) flop per (query, key) pair against 1152 gathered bytes.
-#include "dsa_common.h"
+#include "mla_tile.h"
 
 namespace {
+using namespace mla;
 
-constexpr int DQK = 576;
-constexpr int DV = 512;
-constexpr int BI = 32;                       // keys per tile
-constexpr int TILE_BYTES = BI * DQK * 2;     // 36864
-constexpr int GRP_BYTES = BI * 128;          // one 128-byte group of every key in the tile
-constexpr int KSTEPS = DQK / 16;             // 36
 constexpr int DTILES = DV / 32;              // 16
-constexpr float LOG2E = 1.4426950408889634f;
-
-// 16-byte slot swizzle of key row r inside its 128-byte group: conflict-free for the 128-bit row
-// reads (16 lanes) and for the transpose reads (32 lanes) of this kernel.
-__device__ __forceinline__ int swz(int r) {
-  return (((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1) | ((r ^ (r >> 3)) & 1);
-}
-
-__device__ __forceinline__ void dma16(unsigned lds_base, unsigned goff, const void* gbase) {
-  // Each lane fetches 16 bytes at gbase + goff; the wave's 64 chunks land at lds_base + 16*lane.
-  // (m0 carries the LDS base; nothing else in these kernels uses m0)
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :: "s"(lds_base), "v"(goff), "s"(gbase) : "memory");
-}
 
 // S^T MFMAs are issued through inline asm so that their accumulator lives in architectural VGPRs:
 // the 256 accumulation registers are exactly the O^T accumulators, and a 17th accumulator tuple
@@ -80,37 +61,7 @@ __device__ __forceinline__ void fwd_query(
   int* ntile_s = tlist + NT;
 
   // ---- stage the ids, mark valid slots, list the tiles that have any ---------------------
-  for (int t0 = tid; t0 < K; t0 += 8 * 256) {     // eight loads in flight per thread
-    int v[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = t0 + i * 256 < K ? ids[(size_t)qi * K + t0 + i * 256] : -1;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const bool ok = (v[i] >= 0) && (v[i] < Skv) && (v[i] <= qpos);
-      if (t0 + i * 256 < K) idx_s[t0 + i * 256] = ok ? v[i] : -1;
-    }
-  }
-  __syncthreads();
-  for (int t2 = wave; t2 * 2 < NT; t2 += 4) {
-    int e = t2 * 64 + lane;
-    bool ok = idx_s[e] >= 0;
-    unsigned long long b = __ballot(ok);
-    if (lane == 0) { tmask[2 * t2] = (unsigned)b; tmask[2 * t2 + 1] = (unsigned)(b >> 32); }
-  }
-  __syncthreads();
-  if (wave == 0) {
-    int base = 0;
-    for (int t0 = 0; t0 < NT; t0 += 64) {
-      int t = t0 + lane;
-      bool nz = t < NT && tmask[t] != 0u;
-      unsigned long long b = __ballot(nz);
-      if (nz) tlist[base + __popcll(b & ((1ull << lane) - 1ull))] = t;
-      base += __popcll(b);
-    }
-    if (lane == 0) *ntile_s = base;
-  }
-  __syncthreads();
-  const int ntiles = *ntile_s;
+  const int ntiles = stage_ids(ids, qi, K, Skv, qpos, idx_s, tmask, tlist, ntile_s);
 
   // ---- this wave's Q slice as the B operand of S^T = KV . Q^T ---------------------------
   const int h = wave * 32 + r;
@@ -145,40 +96,12 @@ __device__ __forceinline__ void fwd_query(
     }
   }
 
-  // ---- gather: thread (key = tid/8, sub = tid%8) moves slot `sub` of each of the 9 groups ----
+  // ---- gather of tile n of the list into ring slot n % STAGES; lane-dependent LDS offsets ----
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
-  const int gkey = tid >> 3, gsub = tid & 7;
-  const unsigned gslot_off = (unsigned)((gsub ^ swz(gkey)) * 16);
-  auto issue = [&](int n) {
-    const int tile = tlist[n];
-    int kid = idx_s[tile * BI + gkey];
-    kid = kid < 0 ? 0 : kid;
-    const unsigned goff = (unsigned)kid * (DQK * 2) + gslot_off;
-    const unsigned lb = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)((n % STAGES) * TILE_BYTES + wave * 1024));
-#pragma unroll
-    for (int grp = 0; grp < 9; grp++) dma16(lb + grp * GRP_BYTES, goff + grp * 128, kv);
-  };
-
-  // lane-dependent LDS offsets (tile-relative)
-  unsigned qk_off[4];   // A operand of S^T: row r, 16-byte chunk c = 2*ks + g  ->  c&7 = 2*(ks&3) + g
-#pragma unroll
-  for (int j = 0; j < 4; j++) qk_off[j] = (unsigned)(r * 128 + (((2 * j + g) ^ swz(r)) << 4));
-  // A operand of O^T: transpose reads; lane (blk = lane/16, ii = lane%16) points at key
-  // 16s + 8t + 4g + ii/4, dv column 32*dt + 16*(blk&1) + 4*(ii&3)
-  unsigned pv_off[2][2][2];   // [s][t][dt&1]
-  {
-    const int blk = lane >> 4, ii = lane & 15;
-    const int cl = 2 * (blk & 1) + ((ii & 3) >> 1), half = ii & 1;
-#pragma unroll
-    for (int s = 0; s < 2; s++)
-#pragma unroll
-      for (int t = 0; t < 2; t++) {
-        const int key = 16 * s + 8 * t + 4 * g + (ii >> 2);
-#pragma unroll
-        for (int par = 0; par < 2; par++)
-          pv_off[s][t][par] = (unsigned)(key * 128 + (((4 * par + cl) ^ swz(key)) << 4) + half * 8);
-      }
-  }
+  auto issue = [&](int n) { gather_tile(kv, idx_s, tlist[n], lds0 + (unsigned)((n % STAGES) * TILE_BYTES)); };
+  const LaneOffsets lo = lane_offsets();
+  const unsigned (&qk_off)[4] = lo.row_off;          // A operand of S^T: row r, 16-byte chunk 2*ks + g
+  const unsigned (&pv_off)[2][2][2] = lo.tr_off;     // A operand of O^T: transpose reads, [s][t][dt & 1]
 
   const float c2 = sm_scale * LOG2E;
   float m_ref = -1e30f, l_run = 0.f;

@@ -126,4 +126,25 @@ __device__ __forceinline__ LaneOffsets lane_offsets() {
   return o;
 }
 
+// ---------------------------------------------------------------------------------------------
+// MFMA through inline asm with explicit register files ("v" architectural, "a" accumulation).
+// Back-to-back MFMAs accumulating into the same registers need no software wait states; whoever
+// reads a finished accumulator with a non-MFMA instruction calls mfma_done first.
+// ---------------------------------------------------------------------------------------------
+#define DSA_MFMA_FN(name, ACC, A, B)                                                              \
+  __device__ __forceinline__ void name##_first(f32x16& acc, const bf16x8& a, const bf16x8& b) {   \
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&" ACC(acc) : A(a), B(b));           \
+  }                                                                                               \
+  __device__ __forceinline__ void name(f32x16& acc, const bf16x8& a, const bf16x8& b) {           \
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+" ACC(acc) : A(a), B(b));           \
+  }
+DSA_MFMA_FN(mfma_v_av, "v", "a", "v")   // acc VGPR, A in AGPR, B in VGPR
+DSA_MFMA_FN(mfma_v_vv, "v", "v", "v")
+DSA_MFMA_FN(mfma_a_vv, "a", "v", "v")
+DSA_MFMA_FN(mfma_a_av, "a", "a", "v")
+#undef DSA_MFMA_FN
+__device__ __forceinline__ void mfma_done_v(f32x16& acc) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(acc)); }
+__device__ __forceinline__ void mfma_done_a(f32x16& acc) { asm volatile("s_nop 15\n\ts_nop 3" : "+a"(acc)); }
+
+
 }  // namespace mla

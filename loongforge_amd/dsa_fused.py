@@ -7,6 +7,11 @@ tensor-parallel all-to-alls of the reference are identities at tensor-parallel s
 present; sequence-chunked pipelining ("chunkpipe") is not supported.  The names
 ``MegatronModule``, ``RotaryEmbedding``, ``DSAIndexerKernel`` and ``build_module`` are module
 attributes, as in the reference, so tests can patch them.
+
+Provenance: the constructor argument lists, the order and keyword arguments of the four
+``build_module`` calls, attribute names and error messages are the reference's (Apache-2.0,
+Copyright Baidu), because its tests/test_dsa_fused.py and Megatron's ``build_module`` fix them; the
+arithmetic behind the modules is this repository's HIP kernels.
 """
 import copy
 import math
@@ -285,6 +290,12 @@ class DSAttentionFused(MegatronModule):
         if softmax_scale is None:
             softmax_scale = 1.0 / math.sqrt(k_channels if k_channels is not None else config.kv_channels)
         self.softmax_scale = softmax_scale
+        # the kernels behind this module take at most 2048 slots per query in the backward (the forward
+        # takes 8192): say so here, not in the middle of loss.backward()
+        topk = getattr(self.config, "dsa_indexer_topk", None)
+        if topk is not None and int(topk) > 2048:
+            raise ValueError("DSAttentionFused: dsa_indexer_topk=%d exceeds the 2048 slots per query the sparse "
+                             "attention backward supports" % int(topk))
         self.sparse_attention = build_module(DSADotProductAttention, config=self.config,
                                              softmax_scale=self.softmax_scale)
         self.attn_sink = None
@@ -325,24 +336,29 @@ class DSAttentionFused(MegatronModule):
             chunk_query = F.pad(chunk_query, [0, 0, 0, pad_size])
         offset = self.pg_collection.tp.rank() * chunk_query.size(0)
 
-        output, p_out = self.sparse_attention(
+        # The logits of the selected slots are needed for one thing only, the head-averaged attention
+        # distribution the indexer is trained towards (dsa_fused.py:903-929 of the reference asks the
+        # kernel for p_out [sq, n, topk] and reduces it with triton_attn_dist).  Here the attention call
+        # returns that distribution itself, recomputed from q, kv and lse, and only when the loss will
+        # be formed: no [sq, n, topk] tensor exists (4.3 GB at 8k tokens, 17 GB at 32k).
+        need_loss = self.training and torch.is_grad_enabled() and not self.skip_topk
+        res = self.sparse_attention(
             chunk_query,
             key,
             topk_indices.unsqueeze(0).int(),
             offset,
             attn_mask_type=attn_mask_type,
             packed_seq_params=packed_seq_params,
-            return_p_out=True,
             attn_sink=self.attn_sink,
+            return_attn_dist=self.num_attention_heads if need_loss else 0,
         )
+        output, main_attn_probs = res if need_loss else (res, None)
         if self.num_attention_heads < self.num_attention_heads_padded:
             output = output[..., : self.num_attention_heads, :]
-            p_out = p_out[:, : self.num_attention_heads, :]
 
-        if self.training and torch.is_grad_enabled() and not self.skip_topk:
+        if need_loss:
             indexer_loss_coeff = getattr(self.config, "dsa_indexer_loss_coeff", 0.0)
-            with torch.no_grad():
-                main_attn_probs = triton_attn_dist(p_out, self.softmax_scale)[:, : index_scores.shape[-1]]
+            main_attn_probs = main_attn_probs[:, : index_scores.shape[-1]]
             index_attn_probs = torch.softmax(index_scores, dim=-1)
             loss = F.kl_div((index_attn_probs + 1e-10).log(), main_attn_probs.float() + 1e-10, reduction="sum")
             indexer_loss = indexer_loss_coeff * loss / sq

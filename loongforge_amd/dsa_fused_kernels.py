@@ -60,12 +60,19 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
     out of ``p_out``, which is then [sq, n, topk - window_size]
     (loongforge/models/foundation/deepseek_v4/deepseek_v4_csa.py:2341-2346); attention runs over every
     slot.  As in the reference it is only accepted together with ``return_p_out`` (:2971-2974).
+    ``dist_heads`` > 0 (not in the reference) returns, instead of the logits, what the training path
+    makes of them: the head-averaged attention distribution over the slots, mean over the first
+    ``dist_heads`` heads (dsa_fused.py:915-929), recomputed from q, kv and lse so that no [sq, n, topk]
+    tensor is ever allocated.
     """
 
     @staticmethod
     def forward(ctx, q, kv, indices, chunk_offset=0, sm_scale=None, d_v=512, return_p_out=False,
-                packed_seq_params=None, topk_length=None, attn_sink=None, window_size=0, fast_mode=False):
+                packed_seq_params=None, topk_length=None, attn_sink=None, window_size=0, fast_mode=False,
+                dist_heads=0):
         window_size = int(window_size or 0)
+        if dist_heads and (return_p_out or window_size):
+            raise ValueError("dist_heads replaces return_p_out and does not take a window_size")
         if window_size and not return_p_out:
             raise ValueError("window_size > 0 needs return_p_out=True")
         if window_size % 32:
@@ -92,6 +99,10 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
         if return_p_out:
             ctx.mark_non_differentiable(p_out)
             return out, p_out
+        if dist_heads:
+            dist = ops.attn_dist_qk(q, kv2, ids, lse, chunk_offset, sm_scale, int(dist_heads), attn_sink)
+            ctx.mark_non_differentiable(dist)
+            return out, dist
         return out
 
     @staticmethod
@@ -100,7 +111,7 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
         grad_out = grad_out.squeeze(0).contiguous()
         kv2 = kv.reshape(kv.shape[0], kv.shape[-1])
         grad_q, grad_kv = ops.sparse_mla_bwd(q, kv2, out, grad_out, ids, lse, ctx.chunk_offset, ctx.sm_scale, ctx.d_v)
-        return (grad_q, grad_kv.reshape(kv.shape), None, None, None, None, None, None, None, None, None, None)
+        return (grad_q, grad_kv.reshape(kv.shape), None, None, None, None, None, None, None, None, None, None, None)
 
 
 class DSADotProductAttention(MegatronModule):
@@ -115,7 +126,10 @@ class DSADotProductAttention(MegatronModule):
     def forward(self, query: Tensor, kv: Tensor, indices: Tensor, chunk_offset: int,
                 attn_mask_type: AttnMaskType = None, attention_bias: Tensor = None,
                 packed_seq_params: PackedSeqParams = None, return_p_out: bool = False, window_size: int = 0,
-                topk_length: Optional[Tensor] = None, attn_sink: Optional[Tensor] = None):
+                topk_length: Optional[Tensor] = None, attn_sink: Optional[Tensor] = None,
+                return_attn_dist: int = 0):
+        # return_attn_dist = n > 0 (not in the reference's signature): also return the attention
+        # distribution averaged over the first n heads, [sq, topk] fp32, without materialising p_out
         if attn_mask_type is None:
             attn_mask_type = AttnMaskType.causal
         assert attn_mask_type in (AttnMaskType.causal, AttnMaskType.padding_causal), (
@@ -162,14 +176,16 @@ class DSADotProductAttention(MegatronModule):
 
         res = DSADotProductAttentionFunction.apply(query, kv, indices, chunk_offset, self.softmax_scale, d_v,
                                                    return_p_out, packed_seq_params, topk_length, attn_sink,
-                                                   window_size, True)
-        core_attn_out, p_out = (res if return_p_out else (res, None))
+                                                   window_size, True, int(return_attn_dist))
+        core_attn_out, p_out = (res if (return_p_out or return_attn_dist) else (res, None))
         if qkv_format == "thd":
             core_attn_out = core_attn_out.squeeze(0).contiguous()
         else:
             core_attn_out = core_attn_out.contiguous()
         if return_p_out:
             return core_attn_out, p_out
+        if return_attn_dist:
+            return core_attn_out, p_out[:, :topk]
         return core_attn_out
 
 

@@ -430,6 +430,45 @@ def attn_dist(p_out, sm_scale: float):
     return _attn_dist_op(p_out, float(sm_scale))
 
 
+@torch.library.custom_op("dsa::attn_dist_qk", mutates_args=())
+def _attn_dist_qk_op(q: torch.Tensor, kv: torch.Tensor, ids: torch.Tensor, lse: torch.Tensor, q_start: int,
+                     sm_scale: float, heads_in_mean: int) -> torch.Tensor:
+    _need_gpu(q)
+    if q.ndim != 3 or q.shape[-1] != 576 or q.dtype != torch.bfloat16:
+        raise ValueError("attn_dist_qk expects q [S,H,576] in bf16")
+    if kv.ndim != 2 or kv.shape[-1] != 576 or kv.dtype != torch.bfloat16:
+        raise ValueError("attn_dist_qk expects kv [Skv,576] in bf16")
+    S, H, _ = q.shape
+    K = ids.shape[1]
+    if ids.shape[0] != S or lse.shape != (S, H):
+        raise ValueError("attn_dist_qk: ids [S,K] and lse [S,H] must match q")
+    q, kv, ids, lse = _c(q), _c(kv), _c(ids.to(torch.int32)), _c(lse.float())
+    target = torch.empty(S, K, dtype=torch.float32, device=q.device)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        _lib.check(lib.dsa_attn_dist_qk(q.data_ptr(), kv.data_ptr(), ids.data_ptr(), lse.data_ptr(), S, H, int(heads_in_mean),
+                                        kv.shape[0], K, int(q_start), float(sm_scale), target.data_ptr(), _stream(q)),
+                   "dsa_attn_dist_qk")
+    return target
+
+
+@_attn_dist_qk_op.register_fake
+def _(q, kv, ids, lse, q_start, sm_scale, heads_in_mean):
+    return q.new_empty(q.shape[0], ids.shape[1], dtype=torch.float32)
+
+
+def attn_dist_qk(q, kv, ids, lse, q_start: int, sm_scale: float, heads_in_mean: Optional[int] = None,
+                 attn_sink: Optional[torch.Tensor] = None):
+    """fp32 ``[S,K]``: the same distribution as ``attn_dist(p_out, sm_scale)`` - mean over the first
+    ``heads_in_mean`` heads of the softmax over slots - recomputed from q, kv and the forward's
+    natural-log ``lse`` instead of from materialised logits.  With an attention sink the forward's
+    lse includes the sink term; the softmax over the slots alone has the log-sum-exp
+    ``lse + log(1 - exp(sink - lse))``, which is what the kernel is given then."""
+    if attn_sink is not None:
+        lse = lse + torch.log1p(-torch.exp(attn_sink.to(lse.dtype).view(1, -1) - lse).clamp(max=1.0 - 1e-7))
+    return _attn_dist_qk_op(q, kv, ids, lse, int(q_start), float(sm_scale), int(heads_in_mean or q.shape[1]))
+
+
 # --------------------------------------------------------------------------------------------
 # rotary position embedding fused with the surrounding copies
 # --------------------------------------------------------------------------------------------

@@ -29,6 +29,7 @@ sparse_mla_bwd          pinned: torch.autograd through the forward restatement, 
                         fp64, dense-attention gradients (SDPA autograd) in the covering case;
                         finite differences with a sink.
 attn_dist, indexer_kl_loss   pinned: closed forms, F.kl_div, analytic special cases.
+attn_dist_from_lse      pinned: equals attn_dist on the forward's logits (softmax = exp(z - logsumexp)).
 indexer_bwd             pinned: autograd through the gathered logits; finite differences.
                         unpinned detail: duplicate / out-of-window id handling of the closed
                         lightning_indexer_bwd wheel.
@@ -355,6 +356,29 @@ def attn_dist(p_out: torch.Tensor, sm_scale: float) -> torch.Tensor:
     """
     z = p_out.float() * sm_scale
     return torch.softmax(z, dim=-1).mean(dim=1)
+
+
+def attn_dist_from_lse(q, kv, idx, lse, q_start: int, sm_scale: float, heads: Optional[int] = None,
+                       dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``target[i,t] = mean_{h<heads} exp(q[i,h].kv[idx[i,t]] * sm_scale - lse[i,h])``, 0 on invalid slots.
+
+    The distribution of :func:`attn_dist` (dsa_fused_kernels.py:1877-1895 applied to the forward's
+    logits, dsa_fused.py:928-929) written from the forward's log-sum-exp: per head
+    ``softmax_t(z)[t] = exp(z_t - logsumexp(z))``.  ``heads`` restricts the mean to the leading
+    heads (the reference slices padded heads off before the call, dsa_fused.py:915-917).
+    """
+    sq, h, _ = q.shape
+    heads = h if heads is None else heads
+    valid = sparse_mla_valid(idx, kv.shape[0], q_start)
+    safe = torch.where(valid, idx.to(torch.int64), torch.zeros_like(idx, dtype=torch.int64))
+    out = torch.zeros(sq, idx.shape[1], dtype=dtype)
+    qf, kvf, lf = q.to(dtype), kv.to(dtype), lse.to(dtype)
+    for s in range(0, sq, 64):
+        e = min(sq, s + 64)
+        z = torch.einsum("mhd,mkd->mhk", qf[s:e, :heads], kvf[safe[s:e]]) * sm_scale
+        p = torch.exp(z - lf[s:e, :heads].unsqueeze(-1)).masked_fill(~valid[s:e].unsqueeze(1), 0.0)
+        out[s:e] = p.mean(dim=1)
+    return out
 
 
 def indexer_kl_loss(index_score_topk, target, coeff: float, sq_norm: int, eps: float = 1e-10):

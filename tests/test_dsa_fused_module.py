@@ -1,7 +1,11 @@
 """Constructor-wiring checks of the fused indexer module: the same two behaviours the reference's
 tests/test_dsa_fused.py pins (order of the four build_module calls with the k-norm epsilon routed
 only to k_norm, falling back to layernorm_epsilon; dense indexer loss rejected before anything is
-built), run against this repository's dsa_fused module."""
+built), run against this repository's dsa_fused module.
+
+Provenance: the first two tests follow the reference's tests/test_dsa_fused.py (Apache-2.0,
+Copyright Baidu; same monkeypatched names, configuration and expected error text), because that
+test is the definition of "drop-in" for this module; the remaining tests are this repository's."""
 from types import SimpleNamespace
 
 import pytest

@@ -289,3 +289,39 @@ def test_argument_errors(gpu):
     out, lse, _ = ops.sparse_mla_fwd(q, big, ids, 1_300_000)
     with pytest.raises(ValueError, match="at most"):
         ops.sparse_mla_bwd(q, big, out, torch.zeros_like(out), ids, lse, 1_300_000)
+
+
+@pytest.mark.parametrize("S,H,K,heads,q_start,skv,seed", [
+    (200, 128, 128, 128, 40, 300, 3),
+    (96, 128, 64, 16, 0, None, 5),          # 16 real heads padded to 128: only they count
+    (70, 64, 192, 64, 0, None, 8),
+])
+def test_attn_dist_from_q_kv_lse_matches_oracle_and_the_logits_path(gpu, S, H, K, heads, q_start, skv, seed):
+    from loongforge_amd import ops
+
+    inp = O.make_mla_inputs(S, H, K, seed=seed, skv=skv, q_start=q_start)
+    idx = inp.idx.clone()
+    idx[5, 3] = -1
+    q, kv, ids = inp.q.to(gpu), inp.kv.to(gpu), idx.to(gpu)
+    out, lse, p_out = ops.sparse_mla_fwd(q, kv, ids, q_start, inp.sm_scale, 512, True, torch.float32)
+    got = ops.attn_dist_qk(q, kv, ids, lse, q_start, inp.sm_scale, heads)
+    _, rl, rp = O.sparse_mla_fwd(inp.q, inp.kv, idx, q_start, inp.sm_scale, 512)
+    ref = O.attn_dist_from_lse(inp.q, inp.kv, idx, rl, q_start, inp.sm_scale, heads)
+    assert (got.cpu() - ref).abs().max().item() <= 2e-5
+    assert (got.cpu() - O.attn_dist(rp[:, :heads], inp.sm_scale)).abs().max().item() <= 2e-5
+    # the route through the materialised logits gives the same distribution
+    via_logits = ops.attn_dist(p_out[:, :heads], inp.sm_scale)
+    assert (got - via_logits).abs().max().item() <= 2e-5
+    assert ((got.sum(-1) - 1.0).abs() <= 1e-4).all() and (got[5, 3] == 0).all()
+
+
+def test_attn_dist_from_q_kv_lse_with_sink_is_the_softmax_over_the_slots(gpu):
+    from loongforge_amd import ops
+
+    inp = O.make_mla_inputs(120, 128, 64, seed=12)
+    sink = torch.linspace(-3, 3, 128)
+    q, kv, ids = inp.q.to(gpu), inp.kv.to(gpu), inp.idx.to(gpu)
+    out, lse, p_out = ops.sparse_mla_fwd(q, kv, ids, 0, inp.sm_scale, 512, True, torch.float32, attn_sink=sink.to(gpu))
+    got = ops.attn_dist_qk(q, kv, ids, lse, 0, inp.sm_scale, 128, attn_sink=sink.to(gpu))
+    _, _, rp = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, 0, inp.sm_scale, 512)
+    assert (got.cpu() - O.attn_dist(rp, inp.sm_scale)).abs().max().item() <= 5e-5

@@ -260,6 +260,23 @@ def test_attn_dist_rows_sum_to_one_and_matches_loop():
         np.testing.assert_allclose(t[i].numpy(), acc / 3, rtol=1e-5, atol=1e-7)
 
 
+def test_attn_dist_from_lse_equals_attn_dist_on_the_logits():
+    sq, h, dqk, dv, K = 30, 6, 16, 8, 8
+    q, kv, idx = _inputs(sq, h, K, dqk, seed=53, q_start=2, skv=40)
+    idx = idx.clone()
+    idx[4, 2] = -1
+    sm = 0.31
+    _, lse, p_out = O.sparse_mla_fwd(q, kv, idx, 2, sm, dv, dtype=torch.float64)
+    a = O.attn_dist(p_out, sm).double()
+    b = O.attn_dist_from_lse(q, kv, idx, lse, 2, sm, dtype=torch.float64)
+    torch.testing.assert_close(a, b, rtol=1e-6, atol=1e-8)          # attn_dist itself evaluates in fp32
+    torch.testing.assert_close(b.sum(-1), torch.ones(sq, dtype=torch.float64), rtol=1e-9, atol=1e-9)
+    # leading heads only: the same as slicing the logits
+    a4 = O.attn_dist(p_out[:, :4], sm).double()
+    b4 = O.attn_dist_from_lse(q, kv, idx, lse, 2, sm, heads=4, dtype=torch.float64)
+    torch.testing.assert_close(a4, b4, rtol=1e-6, atol=1e-8)
+
+
 def test_kl_loss_matches_library_and_special_cases():
     g = torch.Generator().manual_seed(29)
     sc = torch.randn(7, 16, generator=g)
