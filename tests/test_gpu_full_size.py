@@ -189,3 +189,50 @@ def test_packed_32k_pipeline(gpu):
     assert ((dk - rdkv).abs() - (2e-2 + 1e-2 * rdkv.abs())).max().item() <= FP32_DKV_EXCESS_LIMIT
     assert torch.equal(dqm[seld], dq[seld])
     assert torch.isfinite(dkv.float()).all() and torch.isfinite(dq.float()).all()
+
+
+def test_config1_tiny_dsa_forward_at_its_stated_size(gpu):
+    """Config 1: batch 1, seq 1024, causal; 16 query heads, d_qk 576, d_v 512; indexer 4 heads x 64, uniform
+    head weights, top-k 256; bf16 N(0,1) from fixed seeds.  The whole forward - indexer, selection, sparse
+    attention, attention distribution, KL loss - on the oracle (CPU) and through the drop-in wrappers: the
+    selection against the oracle's under the tie rule, everything downstream on the oracle's own ids."""
+    from types import SimpleNamespace
+
+    from loongforge_amd import ops
+    from loongforge_amd.dsa_fused_kernels import DSADotProductAttention, DSAIndexerKernel
+    from loongforge_amd.megatron_compat import AttnMaskType
+    from tests.gpu_util import assert_close, valid_sets_equal_up_to_noise
+
+    S, H, Hi, Di, K = 1024, 16, 4, 64, 256
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(S, H, 576, generator=g).to(torch.bfloat16)
+    kv = torch.randn(S, 576, generator=g).to(torch.bfloat16)
+    iq, ik, w = O.make_indexer_inputs(S, Hi, Di, seed=0, w_uniform=True)
+    sm = 192 ** -0.5
+    ref = O.dsa_forward(q, kv, iq, ik, w, K, sm, n_heads=H)
+
+    sc, ids = DSAIndexerKernel()(iq.to(gpu), ik.to(gpu), w.to(gpu), K, 0, None)
+    assert sc.shape == (S, K) and ids.shape == (S, K)
+    logits = ref["aux"]["logits"]
+    band = 2e-4 * logits[torch.isfinite(logits)].abs().max().item()
+    assert valid_sets_equal_up_to_noise(ids, ref["idx"], logits, band) == 0
+    fin = torch.isfinite(ref["scores"])
+    assert torch.equal(torch.isfinite(sc.cpu()), fin)
+    assert (sc.cpu()[fin] - ref["scores"][fin]).abs().max().item() <= band
+
+    cfg = SimpleNamespace(qk_pos_emb_head_dim=64, v_head_dim=128, kv_lora_rank=512, apply_rope_fusion=False,
+                          num_attention_heads=H, kv_channels=192, num_layers=1)
+    attn = DSADotProductAttention(cfg, softmax_scale=sm)
+    q_pad = torch.nn.functional.pad(q, (0, 0, 0, 128 - H)).to(gpu)            # the module pads the heads to 128
+    ref_ids = ref["idx"].to(gpu)
+    out, p_out = attn(q_pad.unsqueeze(1), kv.to(gpu).unsqueeze(1), ref_ids.unsqueeze(0), 0, AttnMaskType.causal,
+                      return_p_out=True)
+    assert_close(out[0, :, :H], ref["out"], "out")
+    target = ops.attn_dist(p_out[:, :H], sm)
+    assert (target.cpu() - ref["target"]).abs().max().item() <= 2e-3           # the logits pass through bf16
+    out2, target2 = attn(q_pad.unsqueeze(1), kv.to(gpu).unsqueeze(1), ref_ids.unsqueeze(0), 0, AttnMaskType.causal,
+                         return_attn_dist=H)
+    assert torch.equal(out2, out)
+    assert (target2.cpu() - ref["target"]).abs().max().item() <= 5e-5
+    loss = O.indexer_kl_loss(ref["scores"], target2.cpu(), 1.0, S)
+    assert abs(loss.item() - ref["loss"].item()) <= 1e-3 * abs(ref["loss"].item()) + 1e-6

@@ -196,3 +196,63 @@ def test_indexer_front_end_with_fused_rope_matches_the_torch_rope(gpu):
         assert all(p.grad is not None and torch.isfinite(p.grad).all() and p.grad.abs().max() > 0
                    for n, p in fused.named_parameters() if "weights_proj" not in n and "k_norm.bias" not in n)
         fused.zero_grad()
+
+
+def test_index_share_second_layer_reuses_the_first_layers_topk(gpu):
+    """dsa_indexer_topk_freq = 2 (dsa_fused.py:752-778, :839-878 of the reference): layer 1 owns an indexer
+    and publishes its top-k ids in the carrier, layer 2 owns none and attends over layer 1's ids; only
+    the computing layer contributes an indexer loss."""
+    from loongforge_amd import dsa_fused, ops
+    from loongforge_amd.megatron_compat import AttnMaskType, ModuleSpec
+
+    S, H, Hi, Di, K, hid, qlr = 320, 16, 4, 64, 64, 96, 48
+    cfg = _cfg(num_attention_heads=H, hidden_size=hid, q_lora_rank=qlr, dsa_indexer_n_heads=Hi,
+               dsa_indexer_head_dim=Di, dsa_indexer_topk=K, dsa_indexer_loss_coeff=1.0, rope_type="rope",
+               rotary_percent=1.0, rotary_base=10000, init_method=None, layernorm_epsilon=1e-5,
+               dsa_indexer_rotate_activation=True, enable_chunkpipe=False, dsa_indexer_topk_freq=2,
+               dsa_indexer_skip_topk_offset=0, num_layers=2)
+    sub = dsa_fused.DSAttentionFusedSubmodules(indexer=ModuleSpec(
+        module=dsa_fused.DSAIndexerFused,
+        submodules=dsa_fused.DSAIndexerFusedSubmodules(linear_wq_b=_Linear, linear_wk=_Linear, k_norm=_Norm,
+                                                       linear_weights_proj=_Linear)))
+    torch.manual_seed(3)
+    layers = [dsa_fused.DSAttentionFused(cfg, sub, layer_number=n, attn_mask_type=AttnMaskType.causal,
+                                         attention_type="self", k_channels=192) for n in (1, 2)]
+    assert layers[0].indexer is not None and not layers[0].skip_topk
+    assert layers[1].indexer is None and layers[1].skip_topk and layers[1].source_layer == 1
+    for p in layers[0].parameters():
+        if p.ndim == 2:
+            torch.nn.init.normal_(p, std=p.shape[1] ** -0.5)
+    layers = [m.to(gpu).train() for m in layers]
+    g = torch.Generator().manual_seed(4)
+
+    def rnd(*shape):
+        return torch.randn(*shape, generator=g).to(torch.bfloat16).to(gpu)
+
+    x, qr = rnd(S, 1, hid), rnd(S, 1, qlr)
+    carrier = SimpleNamespace()
+    dsa_fused.DSAIndexerLossLoggingHelperFused.tracker.clear()
+    # the skipping layer cannot run before its source layer has
+    with pytest.raises(RuntimeError, match="did not run before"):
+        layers[1](rnd(S, 1, H, 576), rnd(S, 1, 576), None, None, x=x, qr=qr, attn_mask_type=AttnMaskType.causal,
+                  index_share_carrier=SimpleNamespace())
+    q1, k1 = rnd(S, 1, H, 576).requires_grad_(True), rnd(S, 1, 576).requires_grad_(True)
+    out1 = layers[0](q1, k1, None, None, x=x, qr=qr, attn_mask_type=AttnMaskType.causal, index_share_carrier=carrier)
+    ids = carrier.dsa_topk_holder[1]
+    assert ids.shape == (S, K) and set(carrier.dsa_topk_holder) == {1}
+    q2, k2 = rnd(S, 1, H, 576).requires_grad_(True), rnd(S, 1, 576).requires_grad_(True)
+    out2 = layers[1](q2, k2, None, None, x=x, qr=qr, attn_mask_type=AttnMaskType.causal, index_share_carrier=carrier)
+    assert set(carrier.dsa_topk_holder) == {1}                       # the skipping layer publishes nothing
+    assert set(dsa_fused.DSAIndexerLossLoggingHelperFused.tracker) == {1}      # ... and adds no indexer loss
+    # layer 2 attended over layer 1's ids: the same kernel on the same ids gives the same bits
+    qp = torch.nn.functional.pad(q2.detach()[:, 0], (0, 0, 0, 128 - H))
+    ref2, _, _ = ops.sparse_mla_fwd(qp, k2.detach()[:, 0], ids.int(), 0, layers[1].softmax_scale)
+    assert torch.equal(out2[0], ref2[:, :H])
+    ro, _, _ = O.sparse_mla_fwd(q2.detach().cpu()[:, 0], k2.detach().cpu()[:, 0], ids.cpu(), 0, layers[1].softmax_scale, 512)
+    assert_close(out2[0], ro, "out of the sharing layer")
+    dout = rnd(1, S, H, 512)
+    (out1 * dout).sum().backward()
+    (out2 * dout).sum().backward()
+    assert_mla_grads(q2.grad[:, 0], k2.grad[:, 0], q2.detach().cpu()[:, 0], k2.detach().cpu()[:, 0], ids.cpu(),
+                     dout[0].cpu(), 0, layers[1].softmax_scale, "sharing layer:", out=out2[0])
+    assert all(p.grad is not None for n, p in layers[0].named_parameters() if "indexer" in n and "k_norm.bias" not in n)
