@@ -232,6 +232,7 @@ __device__ __forceinline__ bool linear_select_sort(const float* __restrict__ src
     for (int i = 0; i < 8; i++) {
       if (e0 + i * BLOCK < n) keys[e0 + i * BLOCK] = f2key(v[i]);
       if (fabsf(v[i]) < INFINITY) { mn = fminf(mn, v[i]); mx = fmaxf(mx, v[i]); nfin++; }
+      else if (!(v[i] < INFINITY)) mx = INFINITY;   // +inf or NaN: infinite span below, the general path takes the row
     }
   }
 #pragma unroll
@@ -306,6 +307,7 @@ __device__ __forceinline__ bool linear_select_sort_regs(const float* __restrict_
 #pragma unroll
     for (int j = 0; j < 4; j++)
       if (fabsf(v[i][j]) < INFINITY) { mn = fminf(mn, v[i][j]); mx = fmaxf(mx, v[i][j]); nfin++; }
+      else if (!(v[i][j] < INFINITY)) mx = INFINITY;   // +inf or NaN: the general path takes the row
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     mn = fminf(mn, __shfl_xor(mn, o, 64));
@@ -389,7 +391,7 @@ __global__ __launch_bounds__(BLOCK, LEAN ? 4 : 1) void topk_kernel(const float* 
     for (int t = tid; t < Kp2; t += BLOCK) {
       float v = t < n ? src[t] : -INFINITY;
       outv[t] = v;
-      outi[t] = (t < n && v > -INFINITY) ? base_id + t : -1;
+      outi[t] = (t < n && v != -INFINITY) ? base_id + t : -1;
     }
   } else {
     if (STAGED && !sorted) {
@@ -441,7 +443,7 @@ __global__ __launch_bounds__(BLOCK, LEAN ? 4 : 1) void topk_kernel(const float* 
       if (take) {
         float v = key2f(k);
         outv[pos] = v;
-        outi[pos] = v > -INFINITY ? base_id + e : -1;
+        outi[pos] = v != -INFINITY ? base_id + e : -1;
         pos++;
       }
     }

@@ -144,7 +144,7 @@ def test_relative_layout_of_packed_logits(gpu):
         assert torch.isinf(rel[i, n:]).all()
 
 
-@pytest.mark.parametrize("kind", ["normal", "ties", "constant", "outlier", "holes", "short", "two_values"])
+@pytest.mark.parametrize("kind", ["normal", "ties", "constant", "outlier", "holes", "short", "two_values", "plus_inf"])
 @pytest.mark.parametrize("K,sorted_out", [(2048, True), (1000, True), (256, True), (512, False)])
 def test_topk_rule_on_crafted_rows(gpu, kind, K, sorted_out):
     """The selection rule on rows that exercise every branch of the kernel: the K largest values, ties
@@ -166,6 +166,9 @@ def test_topk_rule_on_crafted_rows(gpu, kind, K, sorted_out):
         x[torch.rand(rows, n, generator=g) < 0.3] = float("-inf")
     elif kind == "two_values":
         x = (x > 0.5).float()
+    elif kind == "plus_inf":
+        x[:, 5] = float("inf")                            # +inf is the largest value, as for torch.topk
+        x[::2, 4000] = float("inf")
     end = torch.full((rows,), n, dtype=torch.int32)
     if kind == "short":
         end = torch.tensor([1, 2, 63, 64, 255, 256, 257, 999, 1000, 1001, 2047, 2049], dtype=torch.int32)
@@ -176,7 +179,7 @@ def test_topk_rule_on_crafted_rows(gpu, kind, K, sorted_out):
         row = x[i, : int(end[i])].clone()
         row[: int(beg[i])] = float("-inf")                  # columns before the window cannot be selected
         order = torch.sort(-row, stable=True).indices      # descending value, ascending column among equals
-        fin = torch.isfinite(row[order])
+        fin = row[order] > float("-inf")                    # only -inf marks a column that cannot be selected
         exp_ids = order[fin][:K]
         kk = len(exp_ids)
         if sorted_out:
