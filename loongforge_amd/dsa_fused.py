@@ -4,7 +4,11 @@ Counterpart of loongforge/models/common/experimental_attention_variant/dsa_fused
 ``DSAIndexerFused`` (:111) computes indexer q / k / weights and calls ``DSAIndexerKernel``;
 ``DSAttentionFused`` (:718) runs indexer -> sparse attention -> sparse KL indexer loss.  The
 tensor-parallel all-to-alls of the reference are identities at tensor-parallel size 1 and are not
-present; sequence-chunked pipelining ("chunkpipe") is not supported.  The names
+present.  Sequence-chunked pipelining ("chunkpipe", dsa_fused.py:234-421) is supported for the
+unpacked layout: the indexer keys of the earlier chunks of a sequence are kept in a slab, the
+current chunk's queries score ``[cached keys | own keys]`` at their global positions, and the
+gradient a later chunk sends to a cached key is handed to the chunk that produced it when that
+chunk's backward runs.  The names
 ``MegatronModule``, ``RotaryEmbedding``, ``DSAIndexerKernel`` and ``build_module`` are module
 attributes, as in the reference, so tests can patch them.
 
@@ -59,6 +63,47 @@ def rotate_activation(x: torch.Tensor) -> torch.Tensor:
     hidden_size = x.size(-1)
     h = _hadamard(hidden_size, x.device, torch.float32)
     return ((x.float() @ h) * hidden_size ** -0.5).to(x.dtype)
+
+
+class _ChunkKeySlab:
+    """Indexer keys of the chunks of the sequences in flight (dsa_fused.py:240-421).
+
+    Book-keeping of a slab of ``slots * chunksize`` key rows (the rows themselves are a buffer of the
+    module, so that they follow it between devices): a forward micro-batch (= one chunk of one
+    sequence) takes a free slot, the schedule gives it back with ``release``.  ``grads`` collects, per
+    chunk position inside the sequence, the gradient that later chunks' scores send to that chunk's keys.
+    """
+
+    def __init__(self, slots, chunksize):
+        self.slots, self.chunksize = slots, chunksize
+        self.free = list(range(slots))
+        self.slot_of = {}              # forward micro-batch number -> slot
+        self.grads = {}                # chunk position in its sequence -> accumulated gradient
+
+    def rows(self, slot):
+        return slice(slot * self.chunksize, (slot + 1) * self.chunksize)
+
+    def reset(self):
+        self.free = list(range(self.slots))
+        self.slot_of.clear()
+
+    def release(self, micro_batch):
+        slot = self.slot_of.pop(micro_batch, None)
+        if slot is not None:
+            self.free.append(slot)
+
+    def take(self, micro_batch):
+        if not self.free:
+            raise RuntimeError("No available cache chunks for indexer key.")
+        slot = self.free.pop(0)
+        self.slot_of[micro_batch] = slot
+        return self.rows(slot)
+
+    def add_grad(self, position, grad):
+        if position in self.grads:
+            self.grads[position] = self.grads[position] + grad
+        else:
+            self.grads[position] = grad
 
 
 @dataclass
@@ -154,8 +199,102 @@ class DSAIndexerFused(MegatronModule):
             parallel_mode="duplicated",
         )
         if getattr(self.config, "enable_chunkpipe", False):
-            raise NotImplementedError("chunkpipe is not supported by the single-GPU DSA modules")
+            self.setup_chunkpipe_indexer_cache_config()
+            self.init_chunk_indexer_key_cache()
         self.indexer_kernel = DSAIndexerKernel()
+
+    # ---- chunkpipe: the reference's method names (its pipeline schedule calls them) over _ChunkKeySlab ----
+    def setup_chunkpipe_indexer_cache_config(self) -> None:
+        """Slot count of the key slab (dsa_fused.py:240-256): the chunks of one sequence, times the virtual
+        pipeline depth, plus two per later pipeline stage still holding micro-batches in flight."""
+        self.num_chunks_per_seq = self.config.chunk_num_per_seq
+        later_stages = self.pg_collection.pp.size() - self.pg_collection.pp.rank() - 1
+        vpp = getattr(self.config, "virtual_pipeline_model_parallel_size", None)
+        self.indexer_key_cache_chunk_size = 2 * later_stages + self.num_chunks_per_seq * (vpp if vpp is not None else 1)
+
+    def init_chunk_indexer_key_cache(self) -> None:
+        """Allocates the slab next to the module's parameters (dsa_fused.py:289-300)."""
+        par = next(self.parameters(), None)
+        device = par.device if par is not None else torch.device("cpu")
+        dtype = par.dtype if par is not None else torch.bfloat16
+        # the reference sizes its slab by the chunks of one sequence (:293) although its slot numbers run up
+        # to indexer_key_cache_chunk_size (:250-253); the slab here holds every slot
+        self._chunk_slab = _ChunkKeySlab(self.indexer_key_cache_chunk_size, self.config.chunksize)
+        self.register_buffer("indexer_key_cache",
+                             torch.zeros(self.indexer_key_cache_chunk_size * self.config.chunksize,
+                                         self.config.micro_batch_size, self.index_head_dim, device=device, dtype=dtype),
+                             persistent=False)
+
+    @property
+    def indexer_key_cache_grad(self):
+        return self._chunk_slab.grads
+
+    @property
+    def micro_batch_to_cache_chunk_map(self):
+        return self._chunk_slab.slot_of
+
+    @property
+    def empty_chunk_indices(self):
+        return self._chunk_slab.free
+
+    def _require_chunkpipe(self, what):
+        if not getattr(self.config, "enable_chunkpipe", False):
+            raise RuntimeError(what)
+
+    def clear_chunk_indexer_key_cache(self) -> None:
+        self._require_chunkpipe("Chunk indexer key cache operations require chunkpipe to be enabled.")
+        self._chunk_slab.reset()
+
+    def delete_chunk_indexer_key_cache(self, micro_batch_index: int) -> None:
+        self._require_chunkpipe("Chunk indexer key cache operations require chunkpipe to be enabled.")
+        self._chunk_slab.release(micro_batch_index)
+
+    def _chunk_position(self):
+        """Position of the current chunk inside its sequence: the forward counter in a forward pass, the
+        backward counter while a chunk is recomputed for its backward (dsa_fused.py:526-531)."""
+        cfg = self.config
+        mb = cfg.chunkpipe_forward_microbatch if cfg.chunkpipe_forward else cfg.chunkpipe_backward_microbatch
+        return mb, mb % self.num_chunks_per_seq
+
+    def is_enable_grad_chunkpipe(self) -> bool:
+        """Whether this forward will be differentiated (dsa_fused.py:258-287): always when it is the
+        recomputation before a backward; in a plain forward only for the last ``keep_activations_chunks``
+        chunks of a sequence, whose activations are kept, and never in evaluation."""
+        self._require_chunkpipe("This method is valid only for Chunkpipe, please check config.enable_chunkpipe=True")
+        if not self.config.chunkpipe_forward:
+            return True
+        if not self.training:
+            return False
+        pos = self.config.chunkpipe_forward_microbatch % self.num_chunks_per_seq
+        return pos + self.config.keep_activations_chunks >= self.num_chunks_per_seq
+
+    def append_chunk_indexer_key_cache(self, indexer_key: torch.Tensor) -> None:
+        """Keeps this chunk's keys ``[chunksize, b, d]`` for the later chunks of its sequence; only in a forward
+        pass and not for the last chunk, which nobody follows (dsa_fused.py:329-361)."""
+        if not getattr(self.config, "enable_chunkpipe", False) or not self.config.chunkpipe_forward:
+            return
+        mb = self.config.chunkpipe_forward_microbatch
+        if (mb + 1) % self.num_chunks_per_seq == 0:
+            return
+        self.indexer_key_cache[self._chunk_slab.take(mb)] = indexer_key.detach().to(self.indexer_key_cache.dtype)
+
+    def concat_cached_chunk_indexer_key(self, indexer_key: torch.Tensor) -> torch.Tensor:
+        """``[keys of the earlier chunks of this sequence | indexer_key]`` along the sequence.  When the pass is
+        differentiated every cached piece is a leaf whose gradient is collected per chunk position
+        (dsa_fused.py:363-421); the producing chunk adds it to its own key gradient."""
+        if not getattr(self.config, "enable_chunkpipe", False):
+            return indexer_key
+        mb, pos = self._chunk_position()
+        slab, track = self._chunk_slab, self.is_enable_grad_chunkpipe()
+        pieces = []
+        for c in range(pos):
+            piece = self.indexer_key_cache[slab.rows(slab.slot_of[mb - pos + c])].to(indexer_key.dtype, copy=True)
+            if track:
+                piece.requires_grad_(True)
+                piece.register_hook(lambda g, c=c: (slab.add_grad(c, g), g)[1])
+            pieces.append(piece)
+        pieces.append(indexer_key)
+        return torch.cat(pieces, dim=0)
 
     def _apply_rope(self, x, rotary_pos_emb, mscale, cu_seqlens, rotary_pos_cos=None, rotary_pos_sin=None):
         """RoPE on the leading ``qk_pos_emb_head_dim`` channels ("PE first", dsa_fused.py:423-487): the fused
@@ -186,10 +325,14 @@ class DSAIndexerFused(MegatronModule):
         qr = qr.detach()
         rotary_seq_len = self.rotary_pos_emb.get_rotary_seq_len(None, None, x, self.config, packed_seq_params)
         packed_seq = packed_seq_params is not None and packed_seq_params.qkv_format == "thd"
-        rotary_pos_emb = self.rotary_pos_emb(rotary_seq_len, offset=0, packed_seq=packed_seq)
+        chunkpipe = getattr(self.config, "enable_chunkpipe", False)
+        pos_emb_offset = self._chunk_position()[1] * self.config.chunksize if chunkpipe else 0
+        rotary_pos_emb = self.rotary_pos_emb(rotary_seq_len, offset=pos_emb_offset, packed_seq=packed_seq)
         mscale = 1.0
         cos = sin = None
         if getattr(self.config, "apply_rope_fusion", False):
+            if chunkpipe:
+                raise NotImplementedError("chunkpipe with apply_rope_fusion: the cached cos / sin tables carry no offset")
             cos, sin = self.rotary_pos_emb.get_cached_cos_sin(rotary_seq_len, dtype=x.dtype, packed_seq=packed_seq)
         if packed_seq_params is not None:
             cu_seqlens_q = packed_seq_params.cu_seqlens_q_padded
@@ -218,6 +361,12 @@ class DSAIndexerFused(MegatronModule):
             q = rotate_activation(q)
             k = rotate_activation(k)
 
+        if chunkpipe and packed_seq_params is None and self.is_enable_grad_chunkpipe() and k.requires_grad:
+            # what the later chunks of the sequence sent to this chunk's keys (their backward ran first) joins
+            # this chunk's own key gradient (dsa_fused.py:606-622)
+            pos, last = self._chunk_position()[1], self.num_chunks_per_seq - 1
+            k.register_hook(lambda g: g if pos == last else g + self._chunk_slab.grads.pop(pos))
+
         weights, _ = self.linear_weights_proj(x)
         weights = weights * self.index_n_heads ** -0.5
         return q, k, weights
@@ -225,15 +374,22 @@ class DSAIndexerFused(MegatronModule):
     def forward(self, x, qr, packed_seq_params: Optional[PackedSeqParams] = None):
         """-> ``(index_score_topk [s, topk], topk_indices [s, topk])`` (dsa_fused.py:640-703)."""
         # the rotation moves into the kernel's quantiser when the kernel offers it (head dim 128, device tensors)
+        chunkpipe = getattr(self.config, "enable_chunkpipe", False)
+        # (with chunkpipe the cached keys are the rotated ones, so the rotation stays outside the kernel)
         fuse = (getattr(self.config, "dsa_indexer_rotate_activation", True) and self.index_head_dim == 128
-                and x.is_cuda and getattr(self.indexer_kernel, "supports_fused_rotate", False))
+                and x.is_cuda and not chunkpipe and getattr(self.indexer_kernel, "supports_fused_rotate", False))
         indexer_query, indexer_key, indexer_weights = self.get_query_key_weight_tensors(x, qr, packed_seq_params,
                                                                                         defer_rotation=fuse)
         if packed_seq_params is None:
             indexer_query = indexer_query.squeeze(1).contiguous()
         indexer_key = indexer_key.squeeze(1).contiguous()
         indexer_weights = indexer_weights.squeeze(1).contiguous()
+        if chunkpipe and packed_seq_params is None:
+            self.append_chunk_indexer_key_cache(indexer_key.unsqueeze(1))
+            indexer_key = self.concat_cached_chunk_indexer_key(indexer_key.unsqueeze(1)).squeeze(1)
         kv_offset = self.pg_collection.tp.rank() * indexer_query.size(0)
+        if chunkpipe:
+            kv_offset += self._chunk_position()[1] * self.config.chunksize
         return self.indexer_kernel(
             indexer_query,
             indexer_key,
@@ -335,6 +491,11 @@ class DSAttentionFused(MegatronModule):
             pad_size = self.num_attention_heads_padded - self.num_attention_heads
             chunk_query = F.pad(chunk_query, [0, 0, 0, pad_size])
         offset = self.pg_collection.tp.rank() * chunk_query.size(0)
+        if getattr(self.config, "enable_chunkpipe", False):
+            # the query chunk sits behind the earlier chunks of its sequence (dsa_fused.py:897-901)
+            mb = (self.config.chunkpipe_forward_microbatch if self.config.chunkpipe_forward
+                  else self.config.chunkpipe_backward_microbatch)
+            offset += (mb % self.config.chunk_num_per_seq) * self.config.chunksize
 
         # The logits of the selected slots are needed for one thing only, the head-averaged attention
         # distribution the indexer is trained towards (dsa_fused.py:903-929 of the reference asks the

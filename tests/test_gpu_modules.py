@@ -256,3 +256,70 @@ def test_index_share_second_layer_reuses_the_first_layers_topk(gpu):
     assert_mla_grads(q2.grad[:, 0], k2.grad[:, 0], q2.detach().cpu()[:, 0], k2.detach().cpu()[:, 0], ids.cpu(),
                      dout[0].cpu(), 0, layers[1].softmax_scale, "sharing layer:", out=out2[0])
     assert all(p.grad is not None for n, p in layers[0].named_parameters() if "indexer" in n and "k_norm.bias" not in n)
+
+
+def test_chunkpipe_chunks_through_the_kernels_match_the_whole_sequence(gpu):
+    """Chunkpipe (dsa_fused.py:234-421, :674-690, :897-901 of the reference) on the HIP path: every chunk of
+    a sequence, given the latent keys of the sequence so far, selects the same keys as the whole sequence in
+    one call (the indexer scores chunk queries against [cached keys | own keys] at their global positions) and
+    produces the same attention rows bit for bit; the indexer's weight gradients, with the chunks' backward
+    passes run last chunk first, agree with the whole-sequence ones."""
+    import copy
+
+    from loongforge_amd import dsa_fused
+    from loongforge_amd.megatron_compat import AttnMaskType, ModuleSpec
+
+    C, cs, H, Hi, Di, K, hid, qlr = 3, 128, 16, 4, 128, 64, 96, 48
+    S = C * cs
+    base = dict(num_attention_heads=H, hidden_size=hid, q_lora_rank=qlr, dsa_indexer_n_heads=Hi,
+                dsa_indexer_head_dim=Di, dsa_indexer_topk=K, dsa_indexer_loss_coeff=1.0, rope_type="rope",
+                rotary_percent=1.0, rotary_base=10000, init_method=None, layernorm_epsilon=1e-5,
+                dsa_indexer_rotate_activation=True)
+    cfg_w = _cfg(enable_chunkpipe=False, **base)
+    cfg_c = _cfg(enable_chunkpipe=True, chunk_num_per_seq=C, chunksize=cs, micro_batch_size=1, chunkpipe_forward=True,
+                 chunkpipe_forward_microbatch=0, chunkpipe_backward_microbatch=0, keep_activations_chunks=C,
+                 virtual_pipeline_model_parallel_size=None, **base)
+    sub = dsa_fused.DSAttentionFusedSubmodules(indexer=ModuleSpec(
+        module=dsa_fused.DSAIndexerFused,
+        submodules=dsa_fused.DSAIndexerFusedSubmodules(linear_wq_b=_Linear, linear_wk=_Linear, k_norm=_Norm,
+                                                       linear_weights_proj=_Linear)))
+    torch.manual_seed(7)
+    whole = dsa_fused.DSAttentionFused(cfg_w, sub, layer_number=1, attn_mask_type=AttnMaskType.causal,
+                                       attention_type="self", k_channels=192)
+    for p in whole.parameters():
+        if p.ndim == 2:
+            torch.nn.init.normal_(p, std=p.shape[1] ** -0.5)
+    whole = whole.to(gpu).train()
+    chunked = dsa_fused.DSAttentionFused(cfg_c, sub, layer_number=1, attn_mask_type=AttnMaskType.causal,
+                                         attention_type="self", k_channels=192).to(gpu).train()
+    chunked.load_state_dict(whole.state_dict())
+    g = torch.Generator().manual_seed(8)
+
+    def rnd(*shape):
+        return torch.randn(*shape, generator=g).to(torch.bfloat16).to(gpu)
+
+    query, key, x, qr, dout = rnd(S, 1, H, 576), rnd(S, 1, 576), rnd(S, 1, hid), rnd(S, 1, qlr), rnd(1, S, H, 512)
+    out_w = whole(query, key, None, None, x=x, qr=qr, attn_mask_type=AttnMaskType.causal)
+    with torch.no_grad():
+        _, ids_w = whole.indexer(x, qr)
+    (out_w * dout).sum().backward()
+
+    outs = []
+    for c in range(C):
+        cfg_c.chunkpipe_forward_microbatch = c
+        rows = slice(c * cs, (c + 1) * cs)
+        outs.append(chunked(query[rows], key[: (c + 1) * cs], None, None, x=x[rows], qr=qr[rows],
+                            attn_mask_type=AttnMaskType.causal))
+        assert torch.equal(outs[-1], out_w[:, rows])
+    for c in reversed(range(C)):
+        (outs[c] * dout[:, c * cs:(c + 1) * cs]).sum().backward()
+    assert not chunked.indexer.indexer_key_cache_grad
+    for (n, pw), pc in zip(whole.named_parameters(), chunked.parameters()):
+        if "k_norm.bias" in n and pw.grad is None:
+            continue
+        # each chunk's loss is normalised by the chunk's length (loss / sq, dsa_fused.py:940), the whole
+        # sequence's by S: C times the gradient.  The key gradient reaches the projections as a sum of bf16
+        # pieces, one per chunk, instead of one bf16 value.
+        scale = pw.grad.abs().max().item()
+        err = (pc.grad / C - pw.grad).abs().max().item()
+        assert err <= 2e-2 * scale, "%s: %.3e against %.3e" % (n, err, scale)
