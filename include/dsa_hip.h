@@ -66,6 +66,28 @@ int dsa_quant_rowwise_e4m3_weights(const void* x, int64_t rows, int cols, void* 
                                    float* weight_scaled, void* stream);
 
 /*
+ * The indexer front end behind its projections in one pass per 128-element row:
+ *   [LayerNorm ->] [RoPE on the leading 64 elements ->] [Hadamard rotation ->] quantiser [-> weight scaling]
+ * Replaces, on the key side, k_norm -> _apply_rope -> rotate_activation at
+ * loongforge/models/common/experimental_attention_variant/dsa_fused.py:583-606 followed by the quantiser
+ * at dsa_fused_kernels.py:2341-2346, and on the query side _apply_rope -> rotate_activation -> quantiser
+ * -> weight_scaled (dsa_fused.py:568-578, :604-606; dsa_fused_kernels.py:2341-2346, :2362).  Every stage
+ * rounds to bf16 where the separate operations do.  The rotary part uses the formula, rounding and cos /
+ * sin indexing of dsa_rope_rows with equal source and destination pairing (0 adjacent pairs, 1 split pairs
+ * (i, i + 32), -1 none): fused_apply_mla_rope(..., pe_first=True), dsa_fused.py:435-451.
+ *   x [rows, 128] bf16, rows = tokens * rows_per_token; position of a row's token: positions[token], or
+ *   token / batch when positions is NULL; cos, sin [max position + 1, 64] bf16 or f32 (cos_sin_f32);
+ *   ln_weight, ln_bias [128] f32 or both NULL (no LayerNorm); rotate != 0 applies the Hadamard rotation.
+ *   Outputs as dsa_rotate_quant_e4m3 (x8 / scale_inv and / or y) and dsa_quant_rowwise_e4m3_weights
+ *   (weights, weight_scaled [rows] f32, or both NULL).
+ */
+int dsa_indexer_front_e4m3(const void* x, int64_t rows, int cols, int rows_per_token, const float* ln_weight,
+                           const float* ln_bias, float ln_eps, const void* cos, const void* sin,
+                           int cos_sin_f32, int pairing, const int32_t* positions, int batch, int rotate,
+                           void* x8, float* scale_inv, void* y, float eps, int pow2, const float* weights,
+                           float factor, float* weight_scaled, void* stream);
+
+/*
  * Lightning-indexer logits:
  *   logits[i, j - base_i] = k_scale[j] * sum_h q_w[i,h] * relu(q8[i,h,:] . k8[j,:]),  ks[i] <= j < ke[i]
  * and -inf for every other column of row i.  base_i = 0 when `relative` == 0 (dense layout, width

@@ -19,6 +19,8 @@ SIGNATURES = {
     "dsa_quant_rowwise_e4m3": (_i, [_vp, _i64, _i, _vp, _vp, _f, _i, _vp]),
     "dsa_rotate_quant_e4m3": (_i, [_vp, _i64, _i, _vp, _vp, _vp, _f, _i, _vp]),
     "dsa_quant_rowwise_e4m3_weights": (_i, [_vp, _i64, _i, _vp, _vp, _f, _i, _i, _vp, _f, _vp, _vp]),
+    "dsa_indexer_front_e4m3": (_i, [_vp, _i64, _i, _i, _vp, _vp, _f, _vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _f, _i,
+                                    _vp, _f, _vp, _vp]),
     "dsa_indexer_logits": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i64, _i, _i, _vp]),
     "dsa_topk": (_i, [_vp, _i, _i64, _vp, _vp, _i, _vp, _i, _i, _vp, _vp, _vp]),
     "dsa_indexer_topk_workspace_bytes": (_sz, [_i, _i, _i]),

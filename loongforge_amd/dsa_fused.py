@@ -371,12 +371,58 @@ class DSAIndexerFused(MegatronModule):
         weights = weights * self.index_n_heads ** -0.5
         return q, k, weights
 
+    def _fused_front_end(self, x, packed_seq_params):
+        """An :class:`IndexerFrontEnd` when key LayerNorm, rotary embedding and rotation can run inside the indexer
+        kernel's quantisers: fused rotary path configured, 128-channel heads with 64 rotary channels first, a k_norm
+        that is a plain LayerNorm (weight, bias, eps), device tensors, no chunkpipe (its key cache holds finished keys)."""
+        cfg, kern = self.config, self.indexer_kernel
+        k_norm = self.k_norm
+        if not (getattr(cfg, "apply_rope_fusion", False) and x.is_cuda and self.index_head_dim == 128
+                and self.qk_pos_emb_head_dim == 64 and getattr(kern, "supports_fused_front_end", False)
+                and not getattr(cfg, "enable_chunkpipe", False)
+                and isinstance(getattr(k_norm, "weight", None), torch.Tensor)
+                and isinstance(getattr(k_norm, "bias", None), torch.Tensor) and hasattr(k_norm, "eps")):
+            return None
+        from .dsa_fused_kernels import IndexerFrontEnd, _token_positions
+        from . import ops
+
+        packed_seq = packed_seq_params is not None and packed_seq_params.qkv_format == "thd"
+        rotary_seq_len = self.rotary_pos_emb.get_rotary_seq_len(None, None, x, cfg, packed_seq_params)
+        cos, sin = self.rotary_pos_emb.get_cached_cos_sin(rotary_seq_len, dtype=x.dtype, packed_seq=packed_seq)
+        pos_q = pos_k = None
+        if packed_seq_params is not None:
+            cu_q = packed_seq_params.cu_seqlens_q_padded
+            cu_q = packed_seq_params.cu_seqlens_q if cu_q is None else cu_q
+            cu_k = packed_seq_params.cu_seqlens_kv_padded
+            cu_k = packed_seq_params.cu_seqlens_kv if cu_k is None else cu_k
+            cp = self.pg_collection.cp
+            pos_q = _token_positions(cu_q, x.shape[0], cp.rank(), cp.size())
+            pos_k = _token_positions(cu_k, x.shape[0], cp.rank(), cp.size())
+        return IndexerFrontEnd(cos=cos.reshape(-1, 64), sin=sin.reshape(-1, 64), pairing=ops.ROPE_SPLIT, positions_q=pos_q,
+                               positions_k=pos_k, batch=1 if packed_seq_params is not None else x.shape[1],
+                               k_norm_eps=float(k_norm.eps))
+
     def forward(self, x, qr, packed_seq_params: Optional[PackedSeqParams] = None):
         """-> ``(index_score_topk [s, topk], topk_indices [s, topk])`` (dsa_fused.py:640-703)."""
-        # the rotation moves into the kernel's quantiser when the kernel offers it (head dim 128, device tensors)
         chunkpipe = getattr(self.config, "enable_chunkpipe", False)
+        rotate = getattr(self.config, "dsa_indexer_rotate_activation", True)
+        front = self._fused_front_end(x, packed_seq_params)
+        if front is not None:
+            # only the projections run here; k_norm, RoPE, rotation and quantisation are one kernel per side
+            x, qr = x.detach(), qr.detach()
+            q, _ = self.linear_wq_b(qr)
+            q = q.view(*q.size()[:-1], self.index_n_heads, self.index_head_dim)
+            k, _ = self.linear_wk(x)
+            weights, _ = self.linear_weights_proj(x)
+            weights = weights * self.index_n_heads ** -0.5
+            if packed_seq_params is None:
+                q = q.squeeze(1)
+            return self.indexer_kernel(
+                q.contiguous(), k.squeeze(1).contiguous(), weights.squeeze(1).contiguous(), self.index_topk,
+                chunk_offset=self.pg_collection.tp.rank() * q.size(0), packed_seq_params=packed_seq_params,
+                rotate=bool(rotate), front=front, k_norm_weight=self.k_norm.weight, k_norm_bias=self.k_norm.bias)
         # (with chunkpipe the cached keys are the rotated ones, so the rotation stays outside the kernel)
-        fuse = (getattr(self.config, "dsa_indexer_rotate_activation", True) and self.index_head_dim == 128
+        fuse = (rotate and self.index_head_dim == 128
                 and x.is_cuda and not chunkpipe and getattr(self.indexer_kernel, "supports_fused_rotate", False))
         indexer_query, indexer_key, indexer_weights = self.get_query_key_weight_tensors(x, qr, packed_seq_params,
                                                                                         defer_rotation=fuse)

@@ -5,6 +5,7 @@ Drop-in counterparts of loongforge/models/common/experimental_attention_variant/
 :2001, ``DSADotProductAttention`` :2115, ``DSAIndexerKernelFunction`` :2287, ``DSAIndexerKernel``
 :2445), backed by the gfx950 HIP kernels instead of DeepGEMM / FlashInfer / FlashMLA / Triton.
 """
+from dataclasses import dataclass
 from typing import Optional
 
 import torch
@@ -233,7 +234,8 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, index_q: Tensor, index_k: Tensor, weights: Tensor, index_topk: int, chunk_offset: int,
-                packed_seq_params: Optional[PackedSeqParams], rotate: bool = False):
+                packed_seq_params: Optional[PackedSeqParams], rotate: bool = False, front: Optional["IndexerFrontEnd"] = None,
+                k_norm_weight: Optional[Tensor] = None, k_norm_bias: Optional[Tensor] = None):
         assert index_q.ndim == 3 and index_k.ndim == 2 and weights.ndim == 2
         seq_q, head, dim = index_q.size()
         seq_k, _dim = index_k.size()
@@ -249,11 +251,22 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
         # rotate: the Hadamard rotation of the indexer front end is applied here, fused with the
         # quantiser (a zero-padded head dimension cannot be rotated after padding: 128 only)
         assert not rotate or dim == 128, "the fused rotation needs head dim 128"
-        quant = ops.rotate_quant_e4m3 if rotate else ops.quant_rowwise_e4m3
-        # weight_scaled = weights * q_scale * softmax_scale comes out of the query's quantiser kernel
-        q_fp8, q_scale, weight_scaled = ops.quant_rowwise_e4m3_weights(q_p, _pad_to(weights.float(), head_p, 1),
-                                                                       softmax_scale, rotate)
-        k_fp8, k_scale = quant(k_p)
+        if front is None:
+            quant = ops.rotate_quant_e4m3 if rotate else ops.quant_rowwise_e4m3
+            # weight_scaled = weights * q_scale * softmax_scale comes out of the query's quantiser kernel
+            q_fp8, q_scale, weight_scaled = ops.quant_rowwise_e4m3_weights(q_p, _pad_to(weights.float(), head_p, 1),
+                                                                           softmax_scale, rotate)
+            k_fp8, k_scale = quant(k_p)
+        else:
+            # index_q / index_k are the projections' outputs: key LayerNorm, rotary embedding and rotation
+            # happen inside the quantiser kernel (a zero-padded head stays zero through all of them)
+            assert dim == 128, "the fused front end needs head dim 128"
+            q_fp8, q_scale, _, weight_scaled = ops.indexer_front_e4m3(
+                q_p, head_p, None, None, 0.0, front.cos, front.sin, front.pairing, front.positions_q, front.batch, rotate,
+                _pad_to(weights.float(), head_p, 1), softmax_scale)
+            k_fp8, k_scale, _, _ = ops.indexer_front_e4m3(
+                k_p, 1, k_norm_weight, k_norm_bias, front.k_norm_eps, front.cos, front.sin, front.pairing,
+                front.positions_k, front.batch, rotate)
 
         if packed_seq_params is None:
             k_start = torch.zeros(seq_q, dtype=torch.int, device=device)
@@ -275,6 +288,9 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
         ctx.index_topk = index_topk
         ctx.shape = (head, dim)
         ctx.in_dtypes = (index_q.dtype, index_k.dtype, weights.dtype)
+        ctx.front = front
+        if front is not None:
+            ctx.front_saved = (k_p, k_norm_weight, k_norm_bias)
         ctx.save_for_backward(q_fp8, k_fp8, q_scale, k_scale, weight_scaled, topk_indices)
         ctx.mark_non_differentiable(topk_indices)
         return index_score_topk, topk_indices
@@ -294,8 +310,47 @@ class DSAIndexerKernelFunction(torch.autograd.Function):
             d_q = (d_q @ h) * 128 ** -0.5
             d_k = (d_k @ h) * 128 ** -0.5
         dq_t, dk_t, dw_t = ctx.in_dtypes
+        d_ln_w = d_ln_b = None
+        front = ctx.front
+        if front is not None:
+            # back through the rotary embedding (its transpose, on bf16 gradients as the separate kernel's
+            # backward sees them) and, on the key side, through the LayerNorm
+            d_q, d_k = d_q.to(torch.bfloat16).contiguous(), d_k.to(torch.bfloat16).contiguous()
+            _rope_q_rows(d_q, front.cos, front.sin, 0, 64, front.pairing, front.positions_q, front.batch, True)
+            _rope_q_rows(d_k.unsqueeze(1), front.cos, front.sin, 0, 64, front.pairing, front.positions_k, front.batch, True)
+            k_in, ln_w, ln_b = ctx.front_saved
+            d_k, d_ln_w, d_ln_b = _layer_norm_backward(d_k.float(), k_in.float(), ln_w.float(), front.k_norm_eps)
+            d_ln_w, d_ln_b = d_ln_w.to(ln_w.dtype), d_ln_b.to(ln_b.dtype)
         return (d_q[:, :head, :dim].to(dq_t), d_k[:, :dim].to(dk_t), d_weights[:, :head].to(dw_t), None, None, None,
-                None)
+                None, None, d_ln_w, d_ln_b)
+
+
+def _layer_norm_backward(dy: Tensor, x: Tensor, weight: Tensor, eps: float):
+    """Gradients of ``y = (x - mean) * rstd * weight + bias`` over the last dimension (fp32)."""
+    mean = x.mean(-1, keepdim=True)
+    xc = x - mean
+    rstd = torch.rsqrt(xc.square().mean(-1, keepdim=True) + eps)
+    xhat = xc * rstd
+    d_w, d_b = (dy * xhat).sum(0), dy.sum(0)
+    dxhat = dy * weight
+    dx = rstd * (dxhat - dxhat.mean(-1, keepdim=True) - xhat * (dxhat * xhat).mean(-1, keepdim=True))
+    return dx, d_w, d_b
+
+
+@dataclass
+class IndexerFrontEnd:
+    """What ``DSAIndexerKernel(..., front=...)`` needs to run the indexer front end inside its quantiser kernels
+    (dsa_fused.py:568-606 of the reference): the rotary tables ``[positions, 64]``, where a rotation pair sits
+    (``ops.ROPE_ADJACENT`` / ``ops.ROPE_SPLIT``), the position of every query / key token (``None``: token //
+    batch) and the key LayerNorm's epsilon (its weight and bias are passed as tensors so that they get gradients)."""
+
+    cos: Tensor
+    sin: Tensor
+    pairing: int
+    positions_q: Optional[Tensor] = None
+    positions_k: Optional[Tensor] = None
+    batch: int = 1
+    k_norm_eps: float = 1e-5
 
 
 class DSAIndexerKernel(torch.nn.Module):
@@ -305,10 +360,15 @@ class DSAIndexerKernel(torch.nn.Module):
     rotation to ``index_q`` / ``index_k`` inside the quantiser kernel instead of before the call."""
 
     supports_fused_rotate = True
+    supports_fused_front_end = True
 
-    def forward(self, index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params, rotate=False):
+    def forward(self, index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params, rotate=False,
+                front=None, k_norm_weight=None, k_norm_bias=None):
+        """``front`` (an extension, :class:`IndexerFrontEnd`): ``index_q`` / ``index_k`` are the outputs of the
+        projections and the key LayerNorm (``k_norm_weight``, ``k_norm_bias``), the rotary embedding and the rotation
+        run inside the quantiser kernels."""
         return DSAIndexerKernelFunction.apply(index_q, index_k, weights, index_topk, chunk_offset, packed_seq_params,
-                                              rotate)
+                                              rotate, front, k_norm_weight, k_norm_bias)
 
 
 # ---------------------------------------------------------------------------------------------------

@@ -99,6 +99,84 @@ def rotate_quant_e4m3(x: torch.Tensor, eps: float = 1e-12, pow2: bool = True, re
     return (x8.view(_FP8), scale_inv, y) if return_rotated else (x8.view(_FP8), scale_inv)
 
 
+@torch.library.custom_op("dsa::indexer_front_e4m3", mutates_args=())
+def _indexer_front_op(x: torch.Tensor, rows_per_token: int, ln_weight: Optional[torch.Tensor],
+                      ln_bias: Optional[torch.Tensor], ln_eps: float, cos: Optional[torch.Tensor],
+                      sin: Optional[torch.Tensor], pairing: int, positions: Optional[torch.Tensor], batch: int,
+                      rotate: bool, weights: Optional[torch.Tensor], factor: float, want_payload: bool,
+                      want_rows: bool, eps: float,
+                      pow2: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    _need_gpu(x)
+    if x.dtype != torch.bfloat16 or x.shape[-1] != 128:
+        raise ValueError("indexer_front_e4m3 expects bf16 rows of 128 elements")
+    x = _c(x)
+    rows = x.numel() // 128
+    if rows % rows_per_token:
+        raise ValueError("indexer_front_e4m3: %d rows are not a multiple of %d rows per token" % (rows, rows_per_token))
+    if (ln_weight is None) != (ln_bias is None):
+        raise ValueError("indexer_front_e4m3: LayerNorm needs weight and bias")
+    f32 = 0
+    if pairing >= 0:
+        if cos is None or sin is None or cos.dtype != sin.dtype or cos.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError("indexer_front_e4m3: cos / sin must both be fp32 or bf16 tables")
+        cos, sin = _c(cos.reshape(-1, cos.shape[-1])), _c(sin.reshape(-1, sin.shape[-1]))
+        if cos.shape[-1] != 64 or sin.shape != cos.shape:
+            raise ValueError("indexer_front_e4m3: cos / sin rows must have 64 entries")
+        f32 = int(cos.dtype == torch.float32)
+        if positions is not None:
+            positions = _c(positions.to(torch.int32))
+            if positions.numel() != rows // rows_per_token:
+                raise ValueError("indexer_front_e4m3: one position per token expected")
+        elif (rows // rows_per_token + batch - 1) // batch > cos.shape[0]:
+            raise ValueError("indexer_front_e4m3: cos / sin tables are shorter than the sequence")
+    if ln_weight is not None:
+        ln_weight, ln_bias = _c(ln_weight.float()), _c(ln_bias.float())
+        if ln_weight.numel() != 128 or ln_bias.numel() != 128:
+            raise ValueError("indexer_front_e4m3: LayerNorm weight and bias must have 128 entries")
+    if weights is not None:
+        if not want_payload or weights.numel() != rows:
+            raise ValueError("indexer_front_e4m3: one weight per row expected, together with the payload")
+        weights = _c(weights.float())
+    dev = x.device
+    x8 = torch.empty(x.shape if want_payload else (0,), dtype=torch.uint8, device=dev)
+    scale_inv = torch.empty(x.shape[:-1] if want_payload else (0,), dtype=torch.float32, device=dev)
+    y = torch.empty(x.shape if want_rows else (0,), dtype=torch.bfloat16, device=dev)
+    w_scaled = torch.empty(x.shape[:-1] if weights is not None else (0,), dtype=torch.float32, device=dev)
+    ptr = lambda t: t.data_ptr() if t is not None and t.numel() else None   # noqa: E731
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.check(lib.dsa_indexer_front_e4m3(
+            x.data_ptr(), rows, 128, int(rows_per_token), ptr(ln_weight), ptr(ln_bias), float(ln_eps),
+            ptr(cos) if pairing >= 0 else None, ptr(sin) if pairing >= 0 else None, f32, int(pairing), ptr(positions),
+            int(batch), int(rotate), ptr(x8), ptr(scale_inv), ptr(y), float(eps), int(pow2), ptr(weights), float(factor),
+            ptr(w_scaled), _stream(x)), "dsa_indexer_front_e4m3")
+    return x8, scale_inv, y, w_scaled
+
+
+@_indexer_front_op.register_fake
+def _(x, rows_per_token, ln_weight, ln_bias, ln_eps, cos, sin, pairing, positions, batch, rotate, weights, factor,
+      want_payload, want_rows, eps, pow2):
+    return (x.new_empty(x.shape if want_payload else (0,), dtype=torch.uint8),
+            x.new_empty(x.shape[:-1] if want_payload else (0,), dtype=torch.float32),
+            x.new_empty(x.shape if want_rows else (0,), dtype=torch.bfloat16),
+            x.new_empty(x.shape[:-1] if weights is not None else (0,), dtype=torch.float32))
+
+
+def indexer_front_e4m3(x: torch.Tensor, rows_per_token: int = 1, ln_weight=None, ln_bias=None, ln_eps: float = 1e-5,
+                       cos=None, sin=None, pairing: int = -1, positions=None, batch: int = 1, rotate: bool = True,
+                       weights=None, factor: float = 1.0, return_payload: bool = True, return_rows: bool = False,
+                       eps: float = 1e-12, pow2: bool = True):
+    """The indexer front end behind its projections in one kernel: bf16 ``[..., 128]`` rows through
+    [LayerNorm] -> [RoPE of the leading 64 elements, ``pairing`` ROPE_ADJACENT / ROPE_SPLIT, -1 none] ->
+    [Hadamard rotation] -> quantiser.  Returns ``(x8, scale_inv, rows, weight_scaled)``; ``rows`` (the bf16
+    values that were quantised) and ``weight_scaled`` (``weights * scale_inv * factor``) are ``None`` unless
+    asked for."""
+    x8, scale_inv, y, ws = _indexer_front_op(x, rows_per_token, ln_weight, ln_bias, ln_eps, cos, sin, pairing, positions,
+                                             batch, rotate, weights, float(factor), return_payload, return_rows, eps, pow2)
+    return (x8.view(_FP8) if return_payload else None, scale_inv if return_payload else None,
+            y if return_rows else None, ws if weights is not None else None)
+
+
 @torch.library.custom_op("dsa::quant_rowwise_e4m3_weights", mutates_args=())
 def _quant_weights_op(x: torch.Tensor, weights: torch.Tensor, factor: float, rotate: bool, eps: float,
                       pow2: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
