@@ -235,6 +235,24 @@ int dsa_attn_dist_qk(const void* q, const void* kv, const int32_t* ids, const fl
                      void* stream);
 
 /*
+ * MLA weight absorption, one head's projection per (token, head) row, read and written in place inside
+ * larger tensors:  c[s, h, n] = sum_k a[s, h, k] * w[h, n, k]   (bf16, fp32 accumulation).
+ * Replaces the two per-head products around the sparse attention call at
+ * loongforge/models/common/experimental_attention_variant/multi_latent_attention.py:1177-1194 / :1304-1316
+ * (q_content = einsum("...hd,hdk->...hk", q_no_pe, k_up), or the TEGroupedLinear linear_kv_up_proj_absorb_q
+ * with its permutes) and :955-974 (core_attn_out = einsum("...hk,hdk->...hd", core_attn_out, v_up), or
+ * linear_kv_up_proj_absorb_output with movedim / transpose), together with the copies that surround them:
+ * `a` may be the no-position columns of the [S, H, 192] query projection and `c` the latent columns of the
+ * [S, H, 576] attention query (k_dim = 128, n_dim = 512, w = W_UK transposed to [H, 512, 128]); or `a` the
+ * attention output [S, H, 512] and `c` the [S, H * 128] input of the output projection (k_dim = 512,
+ * n_dim = 128, w = W_UV [H, 128, 512]).
+ *   a_tok, a_head, c_tok, c_head: strides in elements between tokens / heads (multiples of 8);
+ *   rows of a, c and w start on 16-byte boundaries.
+ */
+int dsa_mla_absorb(const void* a, int64_t a_tok, int64_t a_head, const void* w, void* c, int64_t c_tok,
+                   int64_t c_head, int S, int H, int k_dim, int n_dim, void* stream);
+
+/*
  * Rotary position embedding of the MLA query / key rows, fused with the copies around it.  Per
  * (token, head) the call copies a "main" part of d_main bf16 elements between two strided tensors
  * (main_src NULL: no main part) and rotates a "pe" part of emb_dim bf16 elements, pair by pair:

@@ -553,6 +553,59 @@ class ApplyMLARotaryEmbAbsorbKV(torch.autograd.Function):
         return d_kv, d_emb, None, None, None, None, None, None, None, None
 
 
+class FusedAbsorbRopeQuery(torch.autograd.Function):
+    """The attention query of the absorbed MLA form in one pass over the up-projected query
+    ``q_up [s, (b,) h, 128 + 64]``:  ``query[..., :512] = q_up[..., :128] @ W_UK[h]`` (the key up-projection
+    absorbed into the query, multi_latent_attention.py:1177-1194 of the reference) and ``query[..., 512:] =
+    rope(q_up[..., 128:])`` (its fused_rope_permute_cat, :1196-1204), both written straight into the
+    ``[.., h, 576]`` rows the attention kernel reads: no q_content tensor in head-major layout, no permute, no
+    concatenation.  ``w_uk_t`` is W_UK as ``[h, 512, 128]``."""
+
+    @staticmethod
+    def forward(ctx, q_up, w_uk_t, cos, sin, cu_seqlens_q, cp_rank, cp_size, rotary_interleaved=False):
+        lead = q_up.shape[:-2]
+        nheads, width = q_up.shape[-2], q_up.shape[-1]
+        d_nope, d_out, emb = w_uk_t.shape[2], w_uk_t.shape[1], width - w_uk_t.shape[2]
+        batch = q_up.shape[1] if q_up.ndim == 4 else 1
+        q3 = q_up.reshape(-1, nheads, width)
+        S = q3.shape[0]
+        query = q_up.new_empty(S, nheads, d_out + emb)
+        positions = _token_positions(cu_seqlens_q, S, cp_rank, cp_size)
+        out_pairing = ops.ROPE_ADJACENT if rotary_interleaved else ops.ROPE_SPLIT
+        ops.mla_absorb_into(q3[:, :, :d_nope], w_uk_t, query[:, :, :d_out])
+        ops.rope_rows(q3[:, :, d_nope:], query[:, :, d_out:], cos, sin, ops.ROPE_ADJACENT, out_pairing, False, positions, batch)
+        ctx.save_for_backward(q3, w_uk_t, cos, sin)
+        ctx.args = (positions, batch, out_pairing, d_nope, d_out, emb, q_up.shape)
+        return query.view(*lead, nheads, d_out + emb)
+
+    @staticmethod
+    def backward(ctx, grad):
+        q3, w_uk_t, cos, sin = ctx.saved_tensors
+        positions, batch, out_pairing, d_nope, d_out, emb, shape = ctx.args
+        g3 = grad.reshape(-1, grad.shape[-2], grad.shape[-1])
+        d_up = torch.empty_like(q3)
+        g_c = g3[:, :, :d_out].transpose(0, 1)                                   # [h, S, 512]
+        d_up[:, :, :d_nope] = torch.bmm(g_c, w_uk_t).transpose(0, 1)
+        ops.rope_rows(g3[:, :, d_out:], d_up[:, :, d_nope:], cos, sin, out_pairing, ops.ROPE_ADJACENT, True, positions, batch)
+        d_w = torch.bmm(g_c.transpose(1, 2), q3[:, :, :d_nope].transpose(0, 1)) if ctx.needs_input_grad[1] else None
+        return d_up.view(shape), d_w, None, None, None, None, None, None
+
+
+def fused_absorb_rope_query(q_up, w_uk_t, cos, sin, cu_seqlens_q=None, cp_rank: int = 0, cp_size: int = 1,
+                            rotary_interleaved: bool = False):
+    """``[.., h, 192]`` up-projected query -> ``[.., h, 576]`` attention query (see :class:`FusedAbsorbRopeQuery`)."""
+    return FusedAbsorbRopeQuery.apply(q_up, w_uk_t, cos, sin, cu_seqlens_q, cp_rank, cp_size, rotary_interleaved)
+
+
+def absorb_attention_output(core_attn_out, w_uv):
+    """``[.., h, 512]`` attention output -> ``[.., h * 128]``: the value up-projection applied per head
+    (multi_latent_attention.py:955-975 of the reference: einsum("...hk,hdk->...hd") then flatten), read from
+    the attention kernel's own layout and written in the layout the output projection reads."""
+    lead, nheads = core_attn_out.shape[:-2], core_attn_out.shape[-2]
+    o3 = core_attn_out.reshape(-1, nheads, core_attn_out.shape[-1])
+    return ops.mla_absorb(o3, w_uv).reshape(*lead, nheads * w_uv.shape[1])
+
+
 def fused_apply_mla_rope_for_absorb_kv(kv, k_pos_emb, cos, sin, emb_dim: int, k_dim: int, cu_seqlens_kv=None,
                                        cp_rank: int = 0, cp_size: int = 1, rotary_interleaved: bool = False):
     """Key rows of the absorbed MLA form: copy of ``kv`` plus the rotated, head-shared ``k_pos_emb``

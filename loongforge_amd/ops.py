@@ -642,3 +642,54 @@ def rope_headsum_inverse(grad_pe: torch.Tensor, cos: torch.Tensor, sin: torch.Te
                                                 tokens, heads, int(in_pairing), _stream(grad_pe)),
                    "dsa_rope_headsum_inverse")
     return d_emb
+
+
+# --------------------------------------------------------------------------------------------
+# MLA weight absorption (per-head projections written in place)
+# --------------------------------------------------------------------------------------------
+def mla_absorb_into(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor) -> None:
+    """``c[s, h, :] = a[s, h, :] @ w[h].T`` for bf16 views ``a [S, H, k]``, ``c [S, H, n]`` (any token / head
+    strides that are multiples of 8 elements, unit stride inside a row) and contiguous ``w [H, n, k]`` with
+    ``(k, n)`` = (128, 512) or (512, 128).  Writes into ``c``; no autograd (see :class:`MlaAbsorb`)."""
+    _need_gpu(a, w, c)
+    if a.dtype != torch.bfloat16 or c.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ValueError("mla_absorb expects bf16 tensors")
+    if a.ndim != 3 or c.ndim != 3 or w.ndim != 3 or a.shape[:2] != c.shape[:2] or w.shape != (a.shape[1], c.shape[2], a.shape[2]):
+        raise ValueError("mla_absorb: shapes a %s, w %s, c %s do not fit c[s,h,:] = a[s,h,:] @ w[h].T"
+                         % (tuple(a.shape), tuple(w.shape), tuple(c.shape)))
+    if a.stride(2) != 1 or c.stride(2) != 1:
+        raise ValueError("mla_absorb: rows must be contiguous")
+    w = _c(w)
+    S, H, k = a.shape
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        _lib.check(lib.dsa_mla_absorb(a.data_ptr(), a.stride(0), a.stride(1), w.data_ptr(), c.data_ptr(), c.stride(0),
+                                      c.stride(1), S, H, k, c.shape[2], _stream(a)), "dsa_mla_absorb")
+
+
+class MlaAbsorb(torch.autograd.Function):
+    """``out[s, h, :] = a[s, h, :] @ w[h].T`` through the HIP kernel, written into ``out`` (a view of a larger
+    tensor, returned as is and marked dirty), with the two gradient products as plain library GEMMs."""
+
+    @staticmethod
+    def forward(ctx, a, w, out):
+        mla_absorb_into(a.detach(), w.detach(), out)
+        ctx.save_for_backward(a, w)
+        ctx.mark_dirty(out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        a, w = ctx.saved_tensors
+        g = grad.transpose(0, 1)                       # [H, S, n]
+        d_a = torch.bmm(g, w).transpose(0, 1) if ctx.needs_input_grad[0] else None          # [S, H, k]
+        d_w = torch.bmm(g.transpose(1, 2), a.transpose(0, 1)) if ctx.needs_input_grad[1] else None   # [H, n, k]
+        return d_a, d_w, None
+
+
+def mla_absorb(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Differentiable per-head projection ``a [S, H, k] , w [H, n, k] -> [S, H, n]``; ``out`` may be a view into
+    a larger tensor (for instance the latent columns of the attention query)."""
+    if out is None:
+        out = a.new_empty(a.shape[0], a.shape[1], w.shape[1])
+    return MlaAbsorb.apply(a, w, out)
