@@ -5,6 +5,7 @@ Drop-in counterparts of loongforge/models/common/experimental_attention_variant/
 :2001, ``DSADotProductAttention`` :2115, ``DSAIndexerKernelFunction`` :2287, ``DSAIndexerKernel``
 :2445), backed by the gfx950 HIP kernels instead of DeepGEMM / FlashInfer / FlashMLA / Triton.
 """
+import os
 from dataclasses import dataclass
 from typing import Optional
 
@@ -63,8 +64,9 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
     slot.  As in the reference it is only accepted together with ``return_p_out`` (:2971-2974).
     ``dist_heads`` > 0 (not in the reference) returns, instead of the logits, what the training path
     makes of them: the head-averaged attention distribution over the slots, mean over the first
-    ``dist_heads`` heads (dsa_fused.py:915-929), recomputed from q, kv and lse so that no [sq, n, topk]
-    tensor is ever allocated.
+    ``dist_heads`` heads (dsa_fused.py:915-929): reduced from the logits when those are a small passing
+    allocation (at most DSA_P_OUT_BUDGET_GIB, default 6, GiB), recomputed from q, kv and lse otherwise, so
+    that no large [sq, n, topk] tensor is ever allocated.
     """
 
     @staticmethod
@@ -90,7 +92,12 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
             if attn_sink.numel() != h_q:
                 attn_sink = attn_sink.flatten().repeat_interleave(h_q // attn_sink.numel())
             attn_sink = attn_sink.contiguous().view(h_q).float()
-        out, lse, p_out = ops.sparse_mla_fwd(q, kv2, ids, chunk_offset, sm_scale, d_v, return_p_out,
+        # the head-averaged distribution comes from materialised logits when they are small enough to be a
+        # passing allocation (forward + 0.9 ms, reduction 0.8 ms at 8k tokens x 128 heads x 2048 slots: 4.3 GB),
+        # and is recomputed from q, kv and lse otherwise (2.7 ms, no [sq, n, topk] tensor: 17 GB at 32k tokens)
+        dist_from_logits = (bool(dist_heads) and
+                            sq * q.size(1) * ids.shape[-1] * 2 <= float(os.environ.get("DSA_P_OUT_BUDGET_GIB", "6")) * 2 ** 30)
+        out, lse, p_out = ops.sparse_mla_fwd(q, kv2, ids, chunk_offset, sm_scale, d_v, return_p_out or dist_from_logits,
                                              attn_sink=attn_sink, p_out_skip=window_size)
         ctx.save_for_backward(q, kv, ids, out, lse)
         ctx.sm_scale = sm_scale
@@ -101,7 +108,11 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
             ctx.mark_non_differentiable(p_out)
             return out, p_out
         if dist_heads:
-            dist = ops.attn_dist_qk(q, kv2, ids, lse, chunk_offset, sm_scale, int(dist_heads), attn_sink)
+            if dist_from_logits:
+                dist = ops.attn_dist(p_out[:, :int(dist_heads)], sm_scale)
+                del p_out
+            else:
+                dist = ops.attn_dist_qk(q, kv2, ids, lse, chunk_offset, sm_scale, int(dist_heads), attn_sink)
             ctx.mark_non_differentiable(dist)
             return out, dist
         return out

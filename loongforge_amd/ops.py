@@ -7,6 +7,7 @@ can be used from compiled graphs and carry fake-tensor shape functions.
 
 There is no CPU path and no fallback: tensors must live on a HIP device.
 """
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -445,6 +446,36 @@ def sparse_mla_fwd(q, kv, ids, q_start: int = 0, sm_scale: Optional[float] = Non
     return out, lse, (p_out if return_p_out else None)
 
 
+_BWD_WS = {}      # device index -> workspace kept between calls
+
+
+def _bwd_workspace(full_bytes: int, device):
+    """Workspace of the sparse-MLA backward: ``full_bytes`` lets it take all queries in one sweep (26 GiB at 8k
+    tokens, top-k 2048); given less, the library walks the queries in chunks.  The size is capped by
+    ``DSA_BWD_WORKSPACE_GIB`` when set and by 80 % of the memory that is free, and the buffer is kept per device
+    and reused by later calls (calls that overlap on one device - other streams - must not share it: set
+    ``DSA_BWD_WORKSPACE_CACHE=0``).  Nothing is kept while a HIP graph is being captured."""
+    want = max(int(full_bytes), 256)
+    cap = os.environ.get("DSA_BWD_WORKSPACE_GIB")
+    if cap:
+        want = min(want, max(int(float(cap) * 2 ** 30), 256))
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    kept = _BWD_WS.get(idx)
+    if kept is not None and kept.numel() >= want:
+        return kept, want
+    free, _ = torch.cuda.mem_get_info(idx)
+    free += kept.numel() if kept is not None else 0
+    want = min(want, max(int(free * 0.8), 256))
+    if kept is not None and kept.numel() >= want:
+        return kept, want
+    _BWD_WS.pop(idx, None)
+    del kept
+    ws = torch.empty(want, dtype=torch.uint8, device=device)
+    if os.environ.get("DSA_BWD_WORKSPACE_CACHE", "1") != "0" and not torch.cuda.is_current_stream_capturing():
+        _BWD_WS[idx] = ws
+    return ws, want
+
+
 @torch.library.custom_op("dsa::sparse_mla_bwd", mutates_args=())
 def _mla_bwd_op(q: torch.Tensor, kv: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, ids: torch.Tensor,
                 lse: torch.Tensor, q_start: int, sm_scale: float, d_v: int) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -459,8 +490,7 @@ def _mla_bwd_op(q: torch.Tensor, kv: torch.Tensor, out: torch.Tensor, dout: torc
     dq = torch.empty_like(q)
     dkv = torch.empty_like(kv)
     lib = _lib.load()
-    nbytes = lib.dsa_sparse_mla_bwd_workspace_bytes(S, H, kv.shape[0], K)
-    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
+    ws, nbytes = _bwd_workspace(lib.dsa_sparse_mla_bwd_workspace_bytes(S, H, kv.shape[0], K), q.device)
     with torch.cuda.device(q.device):
         _lib.check(lib.dsa_sparse_mla_bwd(q.data_ptr(), kv.data_ptr(), out.data_ptr(), dout.data_ptr(), ids.data_ptr(),
                                           lse.data_ptr(), S, H, kv.shape[0], K, int(q_start), float(sm_scale),

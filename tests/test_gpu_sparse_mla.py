@@ -270,6 +270,31 @@ def test_backward_chunked_workspace_through_the_c_abi(gpu):
     assert rc == -3 and b"workspace" in lib.dsa_last_error()
 
 
+def test_backward_op_workspace_is_capped_and_kept(gpu, monkeypatch):
+    """ops.sparse_mla_bwd keeps its workspace between calls (one allocation per device, not one per call) and
+    honours DSA_BWD_WORKSPACE_GIB: a cap below the full size makes the library walk the queries in chunks."""
+    from loongforge_amd import _lib, ops
+
+    inp = O.make_mla_inputs(300, 128, 128, seed=8)
+    q, kv, idx, do = inp.q.to(gpu), inp.kv.to(gpu), inp.idx.to(gpu), inp.dout.to(gpu)
+    out, lse, _ = ops.sparse_mla_fwd(q, kv, idx, 0, inp.sm_scale)
+    ops._BWD_WS.clear()
+    dq1, dkv1 = ops.sparse_mla_bwd(q, kv, out, do, idx, lse, 0, inp.sm_scale)
+    kept = ops._BWD_WS[gpu.index or 0]
+    full = _lib.load().dsa_sparse_mla_bwd_workspace_bytes(300, 128, 300, 128)
+    assert kept.numel() == full
+    ops.sparse_mla_bwd(q, kv, out, do, idx, lse, 0, inp.sm_scale)
+    assert ops._BWD_WS[gpu.index or 0] is kept                      # reused, not reallocated
+    ops._BWD_WS.clear()
+    small = _lib.load().dsa_sparse_mla_bwd_workspace_bytes(100, 128, 300, 128)
+    monkeypatch.setenv("DSA_BWD_WORKSPACE_GIB", repr(small / 2 ** 30))
+    dq2, dkv2 = ops.sparse_mla_bwd(q, kv, out, do, idx, lse, 0, inp.sm_scale)
+    assert ops._BWD_WS[gpu.index or 0].numel() <= small + 256 < full
+    assert torch.equal(dq1, dq2)
+    assert (dkv1.float() - dkv2.float()).abs().max().item() <= 2 * 2.0 ** -8 * dkv1.float().abs().max().item()
+    ops._BWD_WS.clear()
+
+
 def test_argument_errors(gpu):
     from loongforge_amd import ops
 
