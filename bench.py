@@ -2,6 +2,7 @@
 """Benchmark of the fused DSA hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py --config {1,3,5}      one timing row for another configuration of BASELINE.json
 
 One step = one pass of the hot path at sequence length 8192 with all inputs resident in HBM:
   * lightning indexer (fp8, 64 heads x 128) + causal top-k 2048        (benchmark config 2)
@@ -76,6 +77,120 @@ def kernel_sources_sha256():
     return h.hexdigest()
 
 
+def timed_ms(torch, fn, reps=5):
+    """Average time of `fn` over `reps` calls after one untimed call (events on the current stream)."""
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def config_row(n):
+    """One JSON line for configuration n of BASELINE.json (1: tiny DSA forward, 3: sparse-MLA forward at
+    4096 tokens, 5: the whole fused path forward + backward on 32768 packed tokens).  Timing rows beside the
+    headline, not the headline: the parity of these configurations is the business of tests/."""
+    import torch
+
+    from loongforge_amd import ops
+    from oracle import dsa_oracle as O
+
+    dev = torch.device("cuda:0")
+    row = {"n_gpus": 1, "data": "synthetic", "dtype": "bf16", "higher_is_better": True, "vs_baseline": None}
+    if n == 3:
+        S3 = 4096
+        inp = O.make_mla_inputs(S3, H, K, seed=0)
+        pairs = int((inp.idx >= 0).sum())
+        q, kv, idx = inp.q.to(dev), inp.kv.to(dev), inp.idx.to(dev)
+        t = timed_ms(torch, lambda: ops.sparse_mla_fwd(q, kv, idx, 0, inp.sm_scale), 10)
+        fl = 2.0 * H * (DQK + DV) * pairs
+        row.update(metric="sparse-MLA forward TFLOP/s, seq 4096, 128 heads, top-k 2048 (config 3)", unit="TFLOP/s",
+                   value=round(fl / t / 1e9, 1), ms_per_step=round(t, 3), frac_of_bf16_mfma_peak=round(fl / t / 1e9 / PEAK_BF16, 4),
+                   config={"workload": "config 3", "pairs": pairs})
+    elif n == 1:
+        S1, H1, K1 = 1024, 16, 256
+        g = torch.Generator().manual_seed(0)
+        q = torch.randn(S1, H1, DQK, generator=g).to(torch.bfloat16)
+        kv = torch.randn(S1, DQK, generator=g).to(torch.bfloat16)
+        iq = torch.randn(S1, 4, 64, generator=g).to(torch.bfloat16)
+        ik = torch.randn(S1, 64, generator=g).to(torch.bfloat16)
+        w = torch.rand(S1, 4, generator=g)
+        sm = 192.0 ** -0.5
+        t0 = time.time()
+        O.dsa_forward(q, kv, iq, ik, w, K1, sm)
+        t_cpu = time.time() - t0
+        # the kernels take 128-wide indexer rows, 32 indexer heads and 128 query heads: zero padding is exact
+        pad = torch.nn.functional.pad
+        qd, kvd = pad(q, (0, 0, 0, 128 - H1)).to(dev), kv.to(dev)
+        iqd, ikd, wd = pad(iq, (0, 64, 0, 28)).to(dev), pad(ik, (0, 64)).to(dev), pad(w, (0, 28)).to(dev)
+        ks, ke = (x.to(dev) for x in O.indexer_window(S1, 0))
+
+        def step():
+            q8, qs, ws = ops.quant_rowwise_e4m3_weights(iqd, wd, 64 ** -0.5)
+            k8, ksc = ops.quant_rowwise_e4m3(ikd)
+            _, ids = ops.indexer_topk(q8, ws, k8, ksc, ks, ke, K1)
+            return ops.sparse_mla_fwd(qd, kvd, ids, 0, sm)
+
+        t = timed_ms(torch, step, 10)
+        row.update(metric="tiny DSA forward tokens/s: indexer 4x64 + top-k 256 + sparse MLA 16 heads, seq 1024 (config 1)",
+                   unit="tokens/s", value=round(S1 / (t * 1e-3), 1), ms_per_step=round(t, 3),
+                   cpu_baseline={"value": round(S1 / t_cpu, 1), "unit": "tokens/s", "cores": os.cpu_count() or 1, "kind": "port",
+                                 "sample": "the whole configuration through the PyTorch oracle (%.2f s)" % t_cpu},
+                   config={"workload": "config 1"})
+    elif n == 5:
+        T = 32768
+        cu = O.make_packed_cu_seqlens(T, 4, 2048, seed=7)
+        iq, ik, w = O.make_indexer_inputs(T, HI, 128, seed=7)
+        ks, ke = (x.to(dev) for x in O.indexer_window(T, 0, cu))
+        iqd, ikd, wd = iq.to(dev), ik.to(dev), w.to(dev)
+        g = torch.Generator(device=dev).manual_seed(7)
+        q = torch.randn(T, H, DQK, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        kv = torch.randn(T, DQK, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        dout = torch.randn(T, H, DV, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        sm = 192.0 ** -0.5
+        parts = {}
+
+        def step():
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+            ev[0].record()
+            q8, qs, ws = ops.quant_rowwise_e4m3_weights(iqd, wd, 128 ** -0.5)
+            k8, ksc = ops.quant_rowwise_e4m3(ikd)
+            sc, ids = ops.indexer_topk(q8, ws, k8, ksc, ks, ke, K)
+            ev[1].record()
+            out, lse, _ = ops.sparse_mla_fwd(q, kv, ids, 0, sm)
+            ev[2].record()
+            target = ops.attn_dist_qk(q, kv, ids, lse, 0, sm, H)          # 17 GB of logits are never materialised
+            scg = sc.detach().requires_grad_(True)
+            O.indexer_kl_loss(scg, target, 1.0, T).backward()
+            gs = torch.where(ids >= 0, scg.grad, torch.zeros_like(sc)).contiguous()
+            ev[3].record()
+            ops.indexer_bwd(gs, q8, k8, ksc, ws, ids)
+            ev[4].record()
+            ops.sparse_mla_bwd(q, kv, out, dout, ids, lse, 0, sm)
+            ev[5].record()
+            torch.cuda.synchronize()
+            names = ["indexer_topk_ms", "mla_fwd_ms", "attn_dist_kl_ms", "indexer_bwd_ms", "mla_bwd_ms"]
+            for i, nm in enumerate(names):
+                parts[nm] = round(ev[i].elapsed_time(ev[i + 1]), 3)
+            return int((ids >= 0).sum())
+
+        step()
+        pairs = step()
+        t = sum(parts.values())
+        row.update(metric="fused DSA forward + backward tokens/s, 32768 packed tokens in 4 documents (config 5)", unit="tokens/s",
+                   value=round(T / (t * 1e-3), 1), ms_per_step=round(t, 3), config={"workload": "config 5", "pairs": pairs,
+                                                                                    "cu_seqlens": cu.tolist()},
+                   mla_fwd_bwd_tflops=round(2.0 * H * (4 * DQK + 3 * DV) * pairs / ((parts["mla_fwd_ms"] + parts["mla_bwd_ms"]) * 1e-3) / 1e12, 1),
+                   **parts)
+    else:
+        raise SystemExit("bench.py --config takes 1, 3 or 5 (2 and 4 are the default run)")
+    print(json.dumps(row))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -84,6 +199,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (reference kernel for scaling the HBM counters)")
+    ap.add_argument("--config", type=int, default=0, help="print one timing row for configuration 1, 3 or 5 instead")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -97,6 +213,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a HIP device", file=sys.stderr)
         sys.exit(1)
+    if args.config:
+        config_row(args.config)
+        return
     lib = _lib.load()
     blib = _lib.load_bench()         # measurement aids: the backward with per-launch timing, plain movers, an MFMA loop
     dev = torch.device("cuda:0")
@@ -233,6 +352,42 @@ def main():
     t_rope = e0.elapsed_time(e1) / 5
     del qc, qpe
 
+    # the "next" rows either side of the path: the indexer front end behind its projections (RoPE + Hadamard rotation +
+    # quantiser [+ key LayerNorm]) as one kernel per side against the separate kernels, and the MLA weight
+    # absorption written straight into the attention layouts against torch.einsum + permute / concatenate
+    from loongforge_amd.dsa_fused_kernels import absorb_attention_output, fused_absorb_rope_query
+    cos2, sin2 = cos_t.view(S, 64).to(torch.bfloat16), sin_t.view(S, 64).to(torch.bfloat16)
+    lnw, lnb = torch.ones(128, device=dev), torch.zeros(128, device=dev)
+
+    def front_fused():
+        ops.indexer_front_e4m3(iq_d, HI, None, None, 0.0, cos2, sin2, ops.ROPE_SPLIT, None, 1, True, w_d, 128 ** -0.5)
+        ops.indexer_front_e4m3(ik_d, 1, lnw, lnb, 1e-5, cos2, sin2, ops.ROPE_SPLIT, None, 1, True)
+
+    def front_staged():
+        pe = iq_d[:, :, :64]
+        ops.rope_rows(pe, pe, cos2, sin2, ops.ROPE_SPLIT, ops.ROPE_SPLIT, False, None, 1)
+        ops.quant_rowwise_e4m3_weights(iq_d, w_d, 128 ** -0.5, True)
+        kn = torch.nn.functional.layer_norm(ik_d.float(), (128,), lnw, lnb, 1e-5).to(torch.bfloat16).unsqueeze(1)
+        pk = kn[:, :, :64]
+        ops.rope_rows(pk, pk, cos2, sin2, ops.ROPE_SPLIT, ops.ROPE_SPLIT, False, None, 1)
+        ops.rotate_quant_e4m3(kn)
+
+    iq_keep = iq_d.clone()                   # the staged rotary kernel works in place
+    t_front = timed_ms(torch, front_fused)
+    t_front_staged = timed_ms(torch, front_staged)
+    iq_d.copy_(iq_keep)
+    del iq_keep
+    q_up = torch.empty(S, H, 192, dtype=torch.bfloat16, device=dev).normal_()
+    w_uk = (torch.empty(H, 128, 512, dtype=torch.bfloat16, device=dev).normal_() * 0.05)
+    w_uv = (torch.empty(H, 128, 512, dtype=torch.bfloat16, device=dev).normal_() * 0.05)
+    w_uk_t = w_uk.transpose(1, 2).contiguous()
+    t_absorb_q = timed_ms(torch, lambda: fused_absorb_rope_query(q_up, w_uk_t, cos_t, sin_t))
+    t_absorb_q_torch = timed_ms(torch, lambda: fused_rope_permute_cat(
+        torch.einsum("shd,hdk->shk", q_up[:, :, :128], w_uk).permute(1, 0, 2).contiguous(), q_up[:, :, 128:], cos_t, sin_t))
+    t_absorb_o = timed_ms(torch, lambda: absorb_attention_output(out, w_uv))
+    t_absorb_o_torch = timed_ms(torch, lambda: torch.einsum("shk,hdk->shd", out, w_uv).flatten(-2, -1).contiguous())
+    del q_up, w_uk, w_uv, w_uk_t
+
     # what plain data movers with the traffic shape of the two bandwidth-bound backward passes reach:
     # as many 1152-byte rows as the dKV pass writes, at scattered positions, beside a streaming read
     # of 0.6 x that size (P, dS, Q, dO); and a streaming read of the rows (the ordered sum).  Source
@@ -347,6 +502,11 @@ def main():
         "nominal": {"note": "the same times priced on S*K pairs and S*S logits, as the reference's own print-outs do",
                     "mla_fwd_bwd_tflops": round(2.0 * H * (4 * DQK + 3 * DV) * S * K / ((t_fwd + t_bwd) * 1e-3) / 1e12, 1),
                     "indexer_topk_fp8_tflops": round(2.0 * HI * 128 * S * S / (t_idx * 1e-3) / 1e12, 1)},
+        "indexer_front_end_ms": {"one_kernel_per_side": round(t_front, 3), "separate_kernels": round(t_front_staged, 3),
+                                 "gbps": round((3.0 * S * HI * 128 + 3.0 * S * 128) / (t_front * 1e-3) / 1e9, 1)},
+        "mla_absorb_ms": {"query_absorb_rope_in_place": round(t_absorb_q, 3), "query_einsum_permute_rope_cat": round(t_absorb_q_torch, 3),
+                          "output_absorb_in_place": round(t_absorb_o, 3), "output_einsum": round(t_absorb_o_torch, 3),
+                          "output_gbps": round(2.0 * S * H * (512 + 128) / (t_absorb_o * 1e-3) / 1e9, 1)},
         "rope_permute_cat_ms": round(t_rope, 3),
         "rope_permute_cat_gbps": round(4.0 * S * H * DQK / (t_rope * 1e-3) / 1e9, 1),
         "wall_s_per_step": round(wall / n, 4),

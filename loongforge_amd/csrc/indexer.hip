@@ -21,7 +21,6 @@ namespace {
 constexpr int D = 128;          // indexer head dim (bytes per fp8 row)
 constexpr int BK = 128;         // keys per LDS tile
 constexpr int TILE_BYTES = BK * D;
-constexpr int IDX_QW = 1;       // queries per wave (one: 122 registers, four waves per SIMD)
 constexpr int QB = 8;           // queries per workgroup
 
 __device__ __forceinline__ int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
@@ -59,14 +58,14 @@ __device__ __forceinline__ float add_halves(float x) {
   return a + b;
 }
 
-template <int NHT, int QW>   // groups of 32 heads; queries per wave (QB / QW waves per workgroup)
-__global__ __launch_bounds__(64 * QB / QW, QW == 1 ? 4 : 2) void indexer_logits_kernel(
+template <int NHT>   // groups of 32 heads
+__global__ __launch_bounds__(64 * QB, 4) void indexer_logits_kernel(
     const unsigned char* __restrict__ q8, const float* __restrict__ q_w, const unsigned char* __restrict__ k8,
     const float* __restrict__ k_scale, const int* __restrict__ ks, const int* __restrict__ ke,
     int S, int Sk, float* __restrict__ logits, long ld, int relative, int q_begin, int q_count) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * TILE_BYTES + 2 * BK * 4];
   constexpr int HI = NHT * 32;
-  constexpr int NWAVE = QB / QW;
+  constexpr int NWAVE = QB;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: window tests below become scalar branches
   const int r = lane & 31, g = lane >> 5;
@@ -83,20 +82,17 @@ __global__ __launch_bounds__(64 * QB / QW, QW == 1 ? 4 : 2) void indexer_logits_
   }
   jlo = max(jlo, 0);
 
-  // this wave's queries
-  int qi[QW], qks[QW], qke[QW];
-  int wlo = 0x7fffffff, whi = 0;                         // union of the wave's windows
-  i32x8 aq[QW][NHT][2];
-  float wq[QW][NHT][16];
-#pragma unroll
-  for (int u = 0; u < QW; u++) {
-    const int i = qb0 + wave * QW + u;
-    const bool live = i < q_end;
-    qi[u] = live ? i : -1;
-    qks[u] = live ? max(ks[i], 0) : 0;
-    qke[u] = live ? min(ke[i], Sk) : 0;
-    if (live) { wlo = min(wlo, qks[u]); whi = max(whi, qke[u]); }
-    const int is = live ? i : qb0;
+  // this wave's query
+  const int i_q = qb0 + wave;
+  const bool live = i_q < q_end;
+  const int qi = live ? i_q : -1;
+  const int qks = live ? max(ks[i_q], 0) : 0;
+  const int qke = live ? min(ke[i_q], Sk) : 0;
+  const int wlo = live ? qks : 0x7fffffff, whi = live ? qke : 0;     // the wave's window
+  i32x8 aq[NHT][2];
+  float wq[NHT][16];
+  {
+    const int is = live ? i_q : qb0;
 #pragma unroll
     for (int t = 0; t < NHT; t++) {
       const unsigned char* row = q8 + ((size_t)is * HI + 32 * t + r) * D + 32 * g;
@@ -104,24 +100,22 @@ __global__ __launch_bounds__(64 * QB / QW, QW == 1 ? 4 : 2) void indexer_logits_
       for (int s = 0; s < 2; s++) {
         const i32x4 lo = *(const i32x4*)(row + 64 * s);
         const i32x4 hi = *(const i32x4*)(row + 64 * s + 16);
-        aq[u][t][s] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        aq[t][s] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       }
       const float* wrow = q_w + (size_t)is * HI + 32 * t + 4 * g;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const f32x4 w4 = *(const f32x4*)(wrow + 8 * j);
 #pragma unroll
-        for (int e = 0; e < 4; e++) wq[u][t][4 * j + e] = w4[e];
+        for (int e = 0; e < 4; e++) wq[t][4 * j + e] = w4[e];
       }
     }
   }
   DSA_WAIT_VMCNT(0);
 #pragma unroll
-  for (int u = 0; u < QW; u++)
+  for (int t = 0; t < NHT; t++)
 #pragma unroll
-    for (int t = 0; t < NHT; t++)
-#pragma unroll
-      for (int s = 0; s < 2; s++) asm volatile("" : "+v"(aq[u][t][s]));
+    for (int s = 0; s < 2; s++) asm volatile("" : "+v"(aq[t][s]));
 
   const int t_lo = jlo / BK, t_hi = (jhi + BK - 1) / BK;      // key tiles [t_lo, t_hi)
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
@@ -167,25 +161,21 @@ __global__ __launch_bounds__(64 * QB / QW, QW == 1 ? 4 : 2) void indexer_logits_
         bk[s] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       }
       const float ksc = ksc_s[c * 32 + r];
+      float part = 0.f;
 #pragma unroll
-      for (int u = 0; u < QW; u++) {
-        if (QW > 1 && (qi[u] < 0 || j0 >= qke[u] || j0 + 32 <= qks[u])) continue;   // scalar
-        float part = 0.f;
+      for (int tt = 0; tt < NHT; tt++) {
+        f32x16 acc;
 #pragma unroll
-        for (int tt = 0; tt < NHT; tt++) {
-          f32x16 acc;
+        for (int e = 0; e < 16; e++) acc[e] = 0.f;
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[tt][0], bk[0], acc, 0, 0, 0, 127, 0, 127);
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[tt][1], bk[1], acc, 0, 0, 0, 127, 0, 127);
 #pragma unroll
-          for (int e = 0; e < 16; e++) acc[e] = 0.f;
-          acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[u][tt][0], bk[0], acc, 0, 0, 0, 127, 0, 127);
-          acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[u][tt][1], bk[1], acc, 0, 0, 0, 127, 0, 127);
-#pragma unroll
-          for (int e = 0; e < 16; e++) part = fmaf(wq[u][tt][e], relu1(acc[e]), part);
-        }
-        part = add_halves(part) * ksc;
-        if (g == 0 && j >= qks[u] && j < qke[u]) {
-          const int col = relative ? j - qks[u] : j;
-          logits[(size_t)(qi[u] - q_begin) * ld + col] = part;
-        }
+        for (int e = 0; e < 16; e++) part = fmaf(wq[tt][e], relu1(acc[e]), part);
+      }
+      part = add_halves(part) * ksc;
+      if (g == 0 && j >= qks && j < qke) {
+        const int col = relative ? j - qks : j;
+        logits[(size_t)(qi - q_begin) * ld + col] = part;
       }
     }
   }
@@ -209,9 +199,8 @@ int dsa_indexer_logits_block(const void* q8, const float* q_w, const void* k8, c
     fill_neg_inf_kernel<<<dim3(2048), dim3(256), 0, st>>>(logits, q_count, (long)ld, width);
     DSA_CHECK_LAUNCH("dsa_indexer_logits(fill)");
   }
-  constexpr int QW = IDX_QW;
-  dim3 grid((q_count + QB - 1) / QB), block(64 * QB / QW);
-#define DSA_IDX_LAUNCH(N) indexer_logits_kernel<N, QW><<<grid, block, 0, st>>>( \
+  dim3 grid((q_count + QB - 1) / QB), block(64 * QB);
+#define DSA_IDX_LAUNCH(N) indexer_logits_kernel<N><<<grid, block, 0, st>>>( \
     (const unsigned char*)q8, q_w, (const unsigned char*)k8, k_scale, ks, ke, S, Sk, logits, (long)ld, relative, q_begin, q_count)
   if (Hi == 32) DSA_IDX_LAUNCH(1);
   else DSA_IDX_LAUNCH(2);
