@@ -14,7 +14,7 @@
 // time, the weights as the MFMA A operand (LDS row reads), the activation rows as the B operand straight
 // from global memory (16 bytes per lane, next block requested before this block's MFMAs).  With C^T in
 // the accumulators a lane owns one output row, so the result leaves in 16-byte pieces.
-#include "dsa_common.h"
+#include "mla_tile.h"
 
 namespace {
 
@@ -24,7 +24,9 @@ template <int K, int N>
 __global__ __launch_bounds__(256, 1) void absorb_kernel(
     const __bf16* __restrict__ a, long a_tok, long a_head, const __bf16* __restrict__ w,
     __bf16* __restrict__ c, long c_tok, long c_head, int S, int H, int splits) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];     // W[h] as [N][K], 16-byte chunks swizzled by row
+  // W[h] in LDS as K / 64 column groups of [N rows][128 bytes]; inside a group the 16-byte chunk c of row n sits in slot
+  // (c & 7) ^ swz(n): the layout of the attention kernels' key tiles, whose 128-bit row reads are bank-conflict free
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int KS = K / 16, NT = N / 32, CH = K / 8;                          // k-steps, output tiles, chunks per row
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, g = lane >> 5;
   const int h = blockIdx.x / splits, part = blockIdx.x % splits;
@@ -34,7 +36,7 @@ __global__ __launch_bounds__(256, 1) void absorb_kernel(
     const uint4* src = (const uint4*)(w + (size_t)h * N * K);
     for (int e = tid; e < N * CH; e += 256) {
       const int n = e / CH, ch = e % CH;
-      *(uint4*)(smem + ((size_t)n * CH + (ch ^ (n & 7))) * 16) = src[e];
+      *(uint4*)(smem + (size_t)(ch >> 3) * (N * 128) + n * 128 + (((ch & 7) ^ mla::swz(n & 31)) << 4)) = src[e];
     }
   }
   __syncthreads();
@@ -59,10 +61,11 @@ __global__ __launch_bounds__(256, 1) void absorb_kernel(
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[e] = 0.f;
       const int n = 32 * nt + r;
-      const unsigned char* wrow = smem + (size_t)n * CH * 16;
+      const unsigned char* wrow = smem + n * 128;
+      const int sw = mla::swz(r);
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
-        const bf16x8 wv = *(const bf16x8*)(wrow + (((2 * ks + g) ^ (n & 7)) << 4));
+        const bf16x8 wv = *(const bf16x8*)(wrow + (ks >> 2) * (N * 128) + ((((2 * ks + g) & 7) ^ sw) << 4));
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv, cur[ks], acc, 0, 0, 0);
       }
       uint4 o[2];
