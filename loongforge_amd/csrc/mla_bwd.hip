@@ -742,7 +742,7 @@ BwdPlan make_plan(int S, int Skv, int K, size_t budget) {
   return p;
 }
 
-constexpr size_t DEFAULT_BUDGET = (size_t)40 << 30;
+constexpr size_t DEFAULT_BUDGET = (size_t)160 << 30;
 
 }  // namespace
 

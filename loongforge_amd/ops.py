@@ -451,14 +451,14 @@ _BWD_WS = {}      # device index -> workspace kept between calls
 
 def _bwd_workspace(full_bytes: int, device):
     """Workspace of the sparse-MLA backward: ``full_bytes`` lets it take all queries in one sweep (26 GiB at 8k
-    tokens, top-k 2048); given less, the library walks the queries in chunks.  The size is capped by
-    ``DSA_BWD_WORKSPACE_GIB`` when set and by 80 % of the memory that is free, and the buffer is kept per device
+    tokens, top-k 2048; 105 GiB at 32k); given less, the library walks the queries in chunks (about 10 % slower at
+    32k tokens in three chunks).  The size is capped by ``DSA_BWD_WORKSPACE_GIB`` (default 48) and by 80 % of the
+    memory that is free, and the buffer is kept per device
     and reused by later calls (calls that overlap on one device - other streams - must not share it: set
     ``DSA_BWD_WORKSPACE_CACHE=0``).  Nothing is kept while a HIP graph is being captured."""
     want = max(int(full_bytes), 256)
-    cap = os.environ.get("DSA_BWD_WORKSPACE_GIB")
-    if cap:
-        want = min(want, max(int(float(cap) * 2 ** 30), 256))
+    cap = os.environ.get("DSA_BWD_WORKSPACE_GIB", "48")
+    want = min(want, max(int(float(cap) * 2 ** 30), 256))
     idx = device.index if device.index is not None else torch.cuda.current_device()
     kept = _BWD_WS.get(idx)
     if kept is not None and kept.numel() >= want:
