@@ -22,26 +22,33 @@
 namespace {
 using namespace mla;
 
-constexpr int PDS_TILE_BYTES = 16384;        // P and dS of one (query, tile): 2 x [4 waves][2][2][32 keys][8 heads] bf16
+constexpr int PDS_TILE_BYTES = 16384;        // P and dS of one (query, tile): 2 x [16 chunk groups][32 keys][8 heads] bf16
 constexpr int PDS_KIND_BYTES = 8192;
 constexpr int ROW_BYTES = DQK * 2;           // one pair row of the dKV buffer
+constexpr int PDS_THREADS = 512;
 
 // ---------------------------------------------------------------------------------------------
 // pass A: P and dS of every (query, tile)
 // ---------------------------------------------------------------------------------------------
-// One workgroup per query, wave w owns heads [32w, 32w+32).  S = Q.KV^T and dP = dO.V^T share the
-// key-row operand read from LDS; Q and dO are the other MFMA operand, resident in registers (Q and
-// half of dO in accumulation registers, which MFMA can read directly).  The accumulators then hold
-// one key per lane and 16 heads per lane, which is the k-vector layout pass C needs, so P and dS go
-// to HBM as 16-byte chunks without any shuffle.
+// One workgroup of eight waves per query; wave w owns heads [16w, 16w+16).  S = Q.KV^T and dP = dO.V^T
+// are 16x16x32 MFMAs with the heads on the rows (Q and dO rows resident in registers, 8 d-values per
+// lane and step) and the 16 keys of a half tile on the columns (key rows read from LDS, one 1 KB read
+// feeding both products).  At under 256 registers per lane two waves share a SIMD.  Measured against
+// four waves of 32 heads with 32x32x16 MFMAs (one wave per SIMD, half the LDS reads): the backward
+// takes 14.5 instead of 15.1 ms; LDS reads (288 KB per tile) and the MFMAs (2176 clocks per tile and
+// SIMD) are then about level.  A lane ends with 4 heads x 2 half tiles; lanes 32 apart trade halves
+// (one v_permlane32_swap per register pair) so that every lane holds one key's 8 heads in the chunk
+// order pass C reads: chunk group 2w + g = heads 16w + {4g .. 4g+3, 8+4g .. 8+4g+3}.
 template <int STAGES>
 __device__ __forceinline__ void pds_body(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
     const __bf16* __restrict__ out, const __bf16* __restrict__ dout, const float* __restrict__ lse,
     unsigned char* __restrict__ pds, int q0, int ql, int H, int Skv, int K, int q_start, float sm_scale,
     unsigned char* smem) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 31, g = lane >> 5;
+  constexpr int KS = DQK / 32, VS = DV / 32;   // 18 and 16 steps of 32 d-values
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int m = lane & 15, kg = lane >> 4;
   const int qi = q0 + ql;
   const int NT = K / BI;
   int* idx_s = (int*)(smem + STAGES * TILE_BYTES);
@@ -49,122 +56,187 @@ __device__ __forceinline__ void pds_body(
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
   float* stat_s = (float*)(ntile_s + 4);       // [2][128]: lse * log2(e), delta
-  const int ntiles = stage_ids(ids, ql, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
-
-  const int h = wave * 32 + r;
+  // All of the query's rows are requested before the ids are staged: one round trip to memory for
+  // both, instead of one after the other.
+  const int h = wave * 16 + m;
   const bool head_ok = h < H;
   const size_t hrow = (size_t)qi * H + (head_ok ? h : 0);
-  bf16x8 qreg[KSTEPS], doreg[VSTEPS];
+  bf16x8 qreg[KS], doreg[VS], oreg[VS];
   {
-    const bf16x8* qp = (const bf16x8*)(q + hrow * DQK) + g;
-    const bf16x8* dp = (const bf16x8*)(dout + hrow * DV) + g;
-    const bf16x8* op = (const bf16x8*)(out + hrow * DV) + g;
+    const bf16x8* qp = (const bf16x8*)(q + hrow * DQK) + kg;
+    const bf16x8* dp = (const bf16x8*)(dout + hrow * DV) + kg;
+    const bf16x8* op = (const bf16x8*)(out + hrow * DV) + kg;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) qreg[ks] = qp[2 * ks];
+    for (int ks = 0; ks < KS; ks++) qreg[ks] = qp[4 * ks];
 #pragma unroll
-    for (int ks = 0; ks < VSTEPS; ks++) doreg[ks] = dp[2 * ks];
-    // delta = rowsum(O . dO): the O rows come in four batches of eight loads, so that a batch costs
-    // one round trip instead of eight (the fences keep the loads of a batch together)
+    for (int ks = 0; ks < VS; ks++) doreg[ks] = dp[4 * ks];
+#pragma unroll
+    for (int ks = 0; ks < VS; ks++) oreg[ks] = op[4 * ks];
+  }
+  const float lse_h = lse[hrow];
+  __builtin_amdgcn_sched_barrier(0);
+  // (the helper is written for four waves; the other four repeat part of its work with equal results)
+  const int ntiles = stage_ids(ids, ql, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
+  // Q and part of dO live in accumulation registers, which MFMA reads directly
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) asm volatile("" : "+a"(qreg[ks]));
+#pragma unroll
+  for (int ks = 0; ks < VS; ks++) {
+    if (ks < 6) asm volatile("" : "+a"(doreg[ks]));
+    else asm volatile("" : "+v"(doreg[ks]));
+  }
+#pragma unroll
+  for (int ks = 0; ks < VS; ks++) asm volatile("" : "+v"(oreg[ks]));
+
+  const unsigned lds0 = (unsigned)(uintptr_t)smem;
+  // transfers of a tile: thread (key, sub) of either half of the workgroup moves 16 bytes of a 128-byte
+  // group of the key's row; waves 0-3 take groups 0-4, waves 4-7 groups 5-8 (a fifth step does nothing)
+  const int hh = wave >> 2;
+  const int gkey = (tid & 255) >> 3, gsub = tid & 7;
+  const unsigned gslot = (unsigned)((gsub ^ swz(gkey)) * 16) + (unsigned)(hh * 5 * 128);
+  unsigned t_goff = 0, t_lb = 0;
+  auto issue_prepare = [&](int n) {
+    const int tile = tlist[n];
+    int kid = idx_s[tile * BI + gkey];
+    kid = kid < 0 ? 0 : kid;
+    t_goff = (unsigned)kid * (DQK * 2) + gslot;
+    t_lb = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)((n % STAGES) * TILE_BYTES + (wave & 3) * 1024 + hh * 5 * GRP_BYTES));
+  };
+  auto issue_step = [&](int i) {
+    if (hh == 0 || i < 4) dma16(t_lb + i * GRP_BYTES, t_goff + i * 128, kv);
+  };
+  for (int n = 0; n < STAGES - 1 && n < ntiles; n++) {
+    issue_prepare(n);
+#pragma unroll
+    for (int i = 0; i < 5; i++) issue_step(i);
+  }
+  // delta = rowsum(O . dO) while the first tiles travel
+  {
     float part = 0.f;
 #pragma unroll
-    for (int b = 0; b < VSTEPS / 8; b++) {
-      bf16x8 o[8];
+    for (int ks = 0; ks < VS; ks++)
 #pragma unroll
-      for (int i = 0; i < 8; i++) o[i] = op[2 * (8 * b + i)];
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < 8; i++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) part = fmaf((float)o[i][e], (float)doreg[8 * b + i][e], part);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+      for (int e = 0; e < 8; e++) part = fmaf((float)oreg[ks][e], (float)doreg[ks][e], part);
+    part += __shfl_xor(part, 16, 64);
     part += __shfl_xor(part, 32, 64);
-    if (g == 0) {
-      stat_s[h] = head_ok ? lse[hrow] * LOG2E : INFINITY;
+    if (kg == 0) {
+      stat_s[h] = head_ok ? lse_h * LOG2E : INFINITY;
       stat_s[128 + h] = head_ok ? part : 0.f;
-    }
-    DSA_WAIT_VMCNT(0);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+a"(qreg[ks]));
-#pragma unroll
-    for (int ks = 0; ks < VSTEPS; ks++) {
-      if (ks < 16) asm volatile("" : "+a"(doreg[ks]));
-      else asm volatile("" : "+v"(doreg[ks]));
     }
   }
   __syncthreads();
-  // accumulator e of a lane is head 32*wave + 8*(e/4) + 4*g + (e%4), for key (lane & 31)
-  float lse2[16], delta[16];
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const f32x4 a = *(const f32x4*)(stat_s + wave * 32 + 8 * j + 4 * g);
-    const f32x4 b = *(const f32x4*)(stat_s + 128 + wave * 32 + 8 * j + 4 * g);
-#pragma unroll
-    for (int e = 0; e < 4; e++) { lse2[4 * j + e] = a[e]; delta[4 * j + e] = b[e]; }
-  }
+  // accumulator i of a lane is head 16*wave + 4*kg + i, for key 16*kt + m
+  const f32x4 lse2 = *(const f32x4*)(stat_s + wave * 16 + 4 * kg);
+  const f32x4 delta = *(const f32x4*)(stat_s + 128 + wave * 16 + 4 * kg);
 
-  const unsigned lds0 = (unsigned)(uintptr_t)smem;
-  const LaneOffsets lo = lane_offsets();
+  // key-row operand of half tile kt and step ks: row 16*kt + m, 16-byte chunk 4*ks + kg of the row
+  unsigned boff[2][2];
+#pragma unroll
+  for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+    for (int par = 0; par < 2; par++) {
+      const int row = 16 * kt + m;
+      boff[kt][par] = (unsigned)(row * 128 + (((4 * par + kg) ^ swz(row)) << 4));
+    }
   const float c2 = sm_scale * LOG2E;
-  auto issue = [&](int n) { gather_tile(kv, idx_s, tlist[n], lds0 + (unsigned)((n % STAGES) * TILE_BYTES)); };
-  for (int n = 0; n < STAGES - 1 && n < ntiles; n++) issue(n);
 
+  f32x4 sacc[2], dpacc[2];
+  // P and dS of the accumulated tile: the lane's 4 heads for its key of either half tile are two
+  // registers (4 bf16) each
+  auto finish = [&](int tile, unsigned mask) {
+    unsigned pw[2][2], dw[2][2];
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++) {
+      const bool valid = (mask >> (16 * kt + m)) & 1u;
+      float pf[4], df[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        pf[i] = valid ? __builtin_amdgcn_exp2f(fmaf(sacc[kt][i], c2, -lse2[i])) : 0.f;
+        df[i] = pf[i] * (dpacc[kt][i] - delta[i]) * sm_scale;
+      }
+      pw[kt][0] = cvt_pk_bf16(pf[0], pf[1]); pw[kt][1] = cvt_pk_bf16(pf[2], pf[3]);
+      dw[kt][0] = cvt_pk_bf16(df[0], df[1]); dw[kt][1] = cvt_pk_bf16(df[2], df[3]);
+    }
+    // lanes 32 apart trade: the lower lane keeps half tile 0 and gets the partner's heads of it, the
+    // upper lane keeps half tile 1.  Afterwards (x[0], x[1]) is the chunk of key 16*(lane/32) + m:
+    // heads 4g .. 4g+3 then 8+4g .. 8+4g+3 of the wave's 16, g = kg & 1.
+#pragma unroll
+    for (int r2 = 0; r2 < 2; r2++) {
+      swap_halves(pw[0][r2], pw[1][r2]);
+      swap_halves(dw[0][r2], dw[1][r2]);
+    }
+    const int key = 16 * (lane >> 5) + m, g = kg & 1;
+    unsigned char* base = pds + ((size_t)ql * NT + tile) * PDS_TILE_BYTES + (size_t)(2 * wave + g) * 512 + key * 16;
+    *(uint4*)base = make_uint4(dw[0][0], dw[0][1], dw[1][0], dw[1][1]);
+    *(uint4*)(base + PDS_KIND_BYTES) = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
+  };
+
+  // Between two barriers every wave runs the MFMAs of one tile and one `finish`; waves 0-3 finish the
+  // tile they just accumulated, waves 4-7 first finish the previous one.  The two waves of a SIMD (w and
+  // w + 4) are thus half a step apart: the arithmetic and stores of one run under the other's MFMAs.
+  int tile = 0;
+  unsigned mask = 0;
   for (int n = 0; n < ntiles; n++) {
-    // operations issued after this tile's gather: 9 per later gather, 4 stores per finished tile
+    // operations a lane issued after this tile's transfers: D per later tile in flight (5 in waves
+    // 0-3, 4 in waves 4-7), 2 stores per finished tile (waves 4-7 are one tile behind with those)
     {
-      const int need = 9 * min(STAGES - 2, ntiles - 1 - n) + 4 * min(n, STAGES - 1);
-      constexpr int FULL = 9 * (STAGES - 2) + 4 * (STAGES - 1);
-      if (need >= FULL) { DSA_WAIT_VMCNT(FULL); }                  // steady state
-      else if (need >= 9 * (STAGES - 2)) { DSA_WAIT_VMCNT(9 * (STAGES - 2)); }   // first tiles: fewer stores behind
-      else if (need >= 9) { DSA_WAIT_VMCNT(9); }                   // last tiles: fewer gathers ahead
-      else { DSA_WAIT_VMCNT(0); }
+      const int ahead = min(STAGES - 2, ntiles - 1 - n);
+      if (hh == 0) {
+        constexpr int D = 5;
+        const int behind = min(n, STAGES - 1);
+        if (ahead == STAGES - 2 && behind == STAGES - 1) { DSA_WAIT_VMCNT(D * (STAGES - 2) + 2 * (STAGES - 1)); }
+        else if (ahead == STAGES - 2) { DSA_WAIT_VMCNT(D * (STAGES - 2)); }
+        else if (ahead >= 1) { DSA_WAIT_VMCNT(D); }
+        else { DSA_WAIT_VMCNT(0); }
+      } else {
+        constexpr int D = 4;             // (their stores of a step come before its transfers)
+        const int behind = min(n - 1, STAGES - 2);
+        if (ahead == STAGES - 2 && behind == STAGES - 2) { DSA_WAIT_VMCNT(D * (STAGES - 2) + 2 * (STAGES - 2)); }
+        else if (ahead == STAGES - 2) { DSA_WAIT_VMCNT(D * (STAGES - 2)); }
+        else if (ahead >= 1) { DSA_WAIT_VMCNT(D); }
+        else { DSA_WAIT_VMCNT(0); }
+      }
     }
     __syncthreads();
-    if (n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
-    const int tile = tlist[n];
-    const unsigned mask = tmask[tile];
+    // the next tile's transfers go out one at a time between the MFMA steps below: issued together they
+    // would hold every wave at the address unit, which takes 64 bytes per clock for the compute unit
+    const bool more = n + STAGES - 1 < ntiles;
+    if (more) issue_prepare(n + STAGES - 1);
+    const int prev_tile = tile;
+    const unsigned prev_mask = mask;
+    tile = __builtin_amdgcn_readfirstlane(tlist[n]);
+    mask = __builtin_amdgcn_readfirstlane(tmask[tile]);
+    if (hh == 1 && n > 0) finish(prev_tile, prev_mask);
+    __builtin_amdgcn_sched_barrier(0);
     const unsigned char* tb = smem + (n % STAGES) * TILE_BYTES;
-
-    f32x16 sacc, dpacc;
-    {
-      bf16x8 f[4];
 #pragma unroll
-      for (int ks = 0; ks < 4; ks++) f[ks] = *(const bf16x8*)(tb + (ks >> 2) * GRP_BYTES + lo.row_off[ks & 3]);
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) { sacc[kt][e] = 0.f; dpacc[kt][e] = 0.f; }
+    {
+      // step j = 2 * ks + kt; FD operand reads in flight
+      constexpr int FD = 4;
+      bf16x8 f[FD];
+#pragma unroll
+      for (int j = 0; j < FD; j++) f[j] = *(const bf16x8*)(tb + ((j >> 1) >> 1) * GRP_BYTES + boff[j & 1][(j >> 1) & 1]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        if (ks == 0) { mfma_v_av_first(sacc, qreg[0], f[0]); mfma_v_av_first(dpacc, doreg[0], f[0]); }
-        else {
-          mfma_v_av(sacc, qreg[ks], f[ks & 3]);
-          if (ks < 16) mfma_v_av(dpacc, doreg[ks], f[ks & 3]);
-          else if (ks < VSTEPS) mfma_v_vv(dpacc, doreg[ks], f[ks & 3]);
+      for (int j = 0; j < 2 * KS; j++) {
+        const int ks = j >> 1, kt = j & 1;
+        sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qreg[ks], f[j % FD], sacc[kt], 0, 0, 0);
+        if (ks < VS) dpacc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(doreg[ks], f[j % FD], dpacc[kt], 0, 0, 0);
+        if (j + FD < 2 * KS) {
+          const int j2 = j + FD, ks2 = j2 >> 1;
+          f[j % FD] = *(const bf16x8*)(tb + (ks2 >> 1) * GRP_BYTES + boff[j2 & 1][ks2 & 1]);
         }
-        if (ks + 4 < KSTEPS) f[ks & 3] = *(const bf16x8*)(tb + ((ks + 4) >> 2) * GRP_BYTES + lo.row_off[ks & 3]);
+        if (j % 7 == 2 && more) issue_step(j / 7);
         __builtin_amdgcn_sched_barrier(0);
       }
-      mfma_done_v(sacc);
-      mfma_done_v(dpacc);
     }
-    const bool valid = (mask >> r) & 1u;
-    bf16x8 pv[2], dsv[2];
-#pragma unroll
-    for (int s = 0; s < 2; s++)
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const int a = 8 * s + e;
-        const float p = valid ? __builtin_amdgcn_exp2f(fmaf(sacc[a], c2, -lse2[a])) : 0.f;
-        const float ds = p * (dpacc[a] - delta[a]) * sm_scale;
-        pv[s][e] = (__bf16)p;
-        dsv[s][e] = (__bf16)ds;
-      }
-    unsigned char* base = pds + ((size_t)ql * NT + tile) * PDS_TILE_BYTES + (size_t)((wave * 2) * 2 + g) * 512 + r * 16;
-#pragma unroll
-    for (int s = 0; s < 2; s++) {
-      *(bf16x8*)(base + s * 1024) = dsv[s];
-      *(bf16x8*)(base + PDS_KIND_BYTES + s * 1024) = pv[s];
-    }
+    if (hh == 0) finish(tile, mask);
     __builtin_amdgcn_sched_barrier(0);
   }
+  if (hh == 1 && ntiles > 0) finish(tile, mask);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -661,7 +733,7 @@ __device__ __forceinline__ RoleSlot role_slot(int b, int nX, int nY) {
   return {nX > nY, n2 + (b - 2 * n2)};
 }
 
-__global__ __launch_bounds__(256, 1) void bwd_pds_kernel(
+__global__ __launch_bounds__(PDS_THREADS, 1) void bwd_pds_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ kv, const int* __restrict__ ids,
     const __bf16* __restrict__ out, const __bf16* __restrict__ dout, const float* __restrict__ lse,
     unsigned char* __restrict__ pds, int q0, int cnt, int H, int Skv, int K, int q_start, float sm_scale) {
@@ -818,7 +890,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(order)");
     const int* sids = sort_ids ? sorted : ids + (size_t)q0 * K;      // row ql belongs to query q0 + ql
     DSA_MARK(1);
-    bwd_pds_kernel<<<dim3(cnt), dim3(256), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out,
+    bwd_pds_kernel<<<dim3(cnt), dim3(PDS_THREADS), smemA, st>>>((const __bf16*)q, (const __bf16*)kv, sids, (const __bf16*)out,
                                                        (const __bf16*)dout, lse, pds, q0, cnt, H, Skv, K, q_start, sm_scale);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(P, dS)");
     DSA_MARK(2);
