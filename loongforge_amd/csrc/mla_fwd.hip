@@ -60,10 +60,8 @@ __device__ __forceinline__ void fwd_query(
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
 
-  // ---- stage the ids, mark valid slots, list the tiles that have any ---------------------
-  const int ntiles = stage_ids(ids, qi, K, Skv, qpos, idx_s, tmask, tlist, ntile_s);
-
-  // ---- this wave's Q slice as the B operand of S^T = KV . Q^T ---------------------------
+  // ---- this wave's Q slice as the B operand of S^T = KV . Q^T, requested before the ids are staged
+  // so that both come back in one round trip to memory ---------------------------------------------
   const int h = wave * 32 + r;
   const bool head_ok = h < H;
   bf16x8 qreg[KSTEPS];
@@ -71,12 +69,16 @@ __device__ __forceinline__ void fwd_query(
     const bf16x8* qp = (const bf16x8*)(q + ((size_t)qi * H + (head_ok ? h : 0)) * DQK) + g;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) qreg[ks] = qp[2 * ks];
-    // the slice must have landed before the gather pipeline starts: the loop below counts
-    // outstanding vector-memory operations by hand
-    DSA_WAIT_VMCNT(0);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+v"(qreg[ks]));
   }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- stage the ids, mark valid slots, list the tiles that have any ---------------------
+  const int ntiles = stage_ids(ids, qi, K, Skv, qpos, idx_s, tmask, tlist, ntile_s);
+  // the slice must have landed before the gather pipeline starts: the loop below counts
+  // outstanding vector-memory operations by hand
+  DSA_WAIT_VMCNT(0);
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+v"(qreg[ks]));
 
   // slots of tiles that are never visited still need their -inf in p_out
   // (p_out holds the slots from p_skip on: its rows are K - p_skip wide)
@@ -99,6 +101,18 @@ __device__ __forceinline__ void fwd_query(
   // ---- gather of tile n of the list into ring slot n % STAGES; lane-dependent LDS offsets ----
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
   auto issue = [&](int n) { gather_tile(kv, idx_s, tlist[n], lds0 + (unsigned)((n % STAGES) * TILE_BYTES)); };
+  // The same gather in nine steps (one 128-byte group of the key rows each), issued between MFMAs:
+  // nine transfers in a row hold the wave until the memory pipeline has taken them all (about 520
+  // clocks per tile of 4200).
+  unsigned g_goff = 0, g_lb = 0;
+  auto gather_prepare = [&](int n) {
+    const int gkey = tid >> 3, gsub = tid & 7;
+    int kid = idx_s[tlist[n] * BI + gkey];
+    kid = kid < 0 ? 0 : kid;
+    g_goff = (unsigned)kid * (DQK * 2) + (unsigned)((gsub ^ swz(gkey)) * 16);
+    g_lb = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)((n % STAGES) * TILE_BYTES + wave * 1024));
+  };
+  auto gather_step = [&](int grp) { dma16(g_lb + grp * GRP_BYTES, g_goff + grp * 128, kv); };
   const LaneOffsets lo = lane_offsets();
   const unsigned (&qk_off)[4] = lo.row_off;          // A operand of S^T: row r, 16-byte chunk 2*ks + g
   const unsigned (&pv_off)[2][2][2] = lo.tr_off;     // A operand of O^T: transpose reads, [s][t][dt & 1]
@@ -115,7 +129,7 @@ __device__ __forceinline__ void fwd_query(
   // S^T of the tile in stage buffer tb.  Operand reads run four k-steps ahead of the MFMAs; the
   // scheduling fences keep that order (and with it the register budget: Q slice 144 + O^T
   // accumulators 256 of 512 per lane).
-  auto qk_tile = [&](const unsigned char* tb, unsigned mask, f32x16& sacc) {
+  auto qk_tile = [&](const unsigned char* tb, unsigned mask, f32x16& sacc, bool gather) {
     bf16x8 a[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) a[ks] = *(const bf16x8*)(tb + (ks >> 2) * GRP_BYTES + qk_off[ks & 3]);
@@ -125,6 +139,7 @@ __device__ __forceinline__ void fwd_query(
       if (ks == 0) mfma_first(sacc, a[0], qreg[0]);
       else mfma_next(sacc, a[ks & 3], qreg[ks]);
       if (ks + 4 < KSTEPS) a[ks & 3] = *(const bf16x8*)(tb + ((ks + 4) >> 2) * GRP_BYTES + qk_off[ks & 3]);
+      if (ks % 7 == 3 && gather) gather_step(ks / 7);          // groups 0 .. 4
       __builtin_amdgcn_sched_barrier(0);
     }
     mfma_chain_done(sacc);
@@ -156,7 +171,7 @@ __device__ __forceinline__ void fwd_query(
       wait_tile(n);
       if (n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
       f32x16 sacc;
-      qk_tile(smem + (n % STAGES) * TILE_BYTES, tmask[tlist[n]], sacc);
+      qk_tile(smem + (n % STAGES) * TILE_BYTES, tmask[tlist[n]], sacc, false);
       m_ref = fmaxf(m_ref, tile_max(sacc));
     }
     __syncthreads();
@@ -166,14 +181,15 @@ __device__ __forceinline__ void fwd_query(
 
   for (int n = 0; n < ntiles; n++) {
     wait_tile(n);
-    if (n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
+    const bool more = n + STAGES - 1 < ntiles;
+    if (more) gather_prepare(n + STAGES - 1);
 
     const int tile = tlist[n];
     const unsigned mask = tmask[tile];
     const unsigned char* tb = smem + (n % STAGES) * TILE_BYTES;
 
     f32x16 sacc;
-    qk_tile(tb, mask, sacc);
+    qk_tile(tb, mask, sacc, more);
     if (POUT != 0 && head_ok && tile * BI >= p_skip) {
       const size_t prow = ((size_t)qi * H + h) * (K - p_skip) + (size_t)(tile * BI - p_skip);
       if (POUT == 2) {
@@ -243,6 +259,7 @@ __device__ __forceinline__ void fwd_query(
               v[dt & 1][s][t] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                   LDS_PTR(i16x4, tb + ((dt + 2) >> 1) * GRP_BYTES + pv_off[s][t][dt & 1]));
         }
+        if (dt % 4 == 1 && more) gather_step(5 + dt / 4);        // groups 5 .. 8
         __builtin_amdgcn_sched_barrier(0);
       }
     }
