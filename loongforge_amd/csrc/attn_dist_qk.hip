@@ -35,8 +35,7 @@ __global__ __launch_bounds__(256, 1) void attn_dist_qk_kernel(
   int* ntile_s = tlist + NT;
   float* part_s = (float*)(ntile_s + 4);
   for (int t = tid; t < 4 * K; t += 256) part_s[t] = 0.f;   // tiles without a valid slot are never visited
-  const int ntiles = stage_ids(ids, qi, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
-
+  // the query's rows are requested before the ids are staged: one round trip to memory for both
   const int h = wave * 32 + r;
   const size_t hrow = (size_t)qi * H + (h < H ? h : 0);
   bf16x8 qreg[KSTEPS];
@@ -44,9 +43,6 @@ __global__ __launch_bounds__(256, 1) void attn_dist_qk_kernel(
     const bf16x8* qp = (const bf16x8*)(q + hrow * DQK) + g;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) qreg[ks] = qp[2 * ks];
-    DSA_WAIT_VMCNT(0);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+a"(qreg[ks]));
   }
   float lse2[16];
 #pragma unroll
@@ -54,6 +50,13 @@ __global__ __launch_bounds__(256, 1) void attn_dist_qk_kernel(
     const int hh = wave * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
     lse2[e] = hh < Hm ? lse[(size_t)qi * H + hh] * LOG2E : INFINITY;
   }
+  __builtin_amdgcn_sched_barrier(0);
+  const int ntiles = stage_ids(ids, qi, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
+  DSA_WAIT_VMCNT(0);
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ks++) asm volatile("" : "+a"(qreg[ks]));
+#pragma unroll
+  for (int e = 0; e < 16; e++) asm volatile("" : "+v"(lse2[e]));
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
   const LaneOffsets lo = lane_offsets();
   const float c2 = sm_scale * LOG2E;
@@ -63,7 +66,18 @@ __global__ __launch_bounds__(256, 1) void attn_dist_qk_kernel(
     const int ahead = min(STAGES - 2, ntiles - 1 - n);      // gathers issued after this tile's: 9 operations each
     if (ahead >= 2) { DSA_WAIT_VMCNT(18); } else if (ahead == 1) { DSA_WAIT_VMCNT(9); } else { DSA_WAIT_VMCNT(0); }
     __syncthreads();
-    if (n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
+    // the next tile's nine transfers go out between the MFMA steps: issued in a row they would hold the
+    // wave until the memory pipeline has taken them all
+    const bool more = n + STAGES - 1 < ntiles;
+    unsigned g_goff = 0, g_lb = 0;
+    if (more) {
+      const int nn = n + STAGES - 1;
+      const int gkey = tid >> 3, gsub = tid & 7;
+      int kid = idx_s[tlist[nn] * BI + gkey];
+      kid = kid < 0 ? 0 : kid;
+      g_goff = (unsigned)kid * (DQK * 2) + (unsigned)((gsub ^ swz(gkey)) * 16);
+      g_lb = __builtin_amdgcn_readfirstlane(lds0 + (unsigned)((nn % STAGES) * TILE_BYTES + wave * 1024));
+    }
     const int tile = tlist[n];
     const unsigned mask = tmask[tile];
     const unsigned char* tb = smem + (n % STAGES) * TILE_BYTES;
@@ -78,6 +92,7 @@ __global__ __launch_bounds__(256, 1) void attn_dist_qk_kernel(
         if (ks == 0) mfma_v_av_first(sacc, qreg[0], f[0]);
         else mfma_v_av(sacc, qreg[ks], f[ks & 3]);
         if (ks + 4 < KSTEPS) f[ks & 3] = *(const bf16x8*)(tb + ((ks + 4) >> 2) * GRP_BYTES + lo.row_off[ks & 3]);
+        if (ks % 4 == 1 && more) dma16(g_lb + (ks / 4) * GRP_BYTES, g_goff + (ks / 4) * 128, kv);
         __builtin_amdgcn_sched_barrier(0);
       }
       mfma_done_v(sacc);
