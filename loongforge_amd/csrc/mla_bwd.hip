@@ -93,7 +93,10 @@ __device__ __forceinline__ void pds_body(
   // group of the key's row; waves 0-3 take groups 0-4, waves 4-7 groups 5-8 (a fifth step does nothing)
   const int hh = wave >> 2;
   const int gkey = (tid & 255) >> 3, gsub = tid & 7;
-  const unsigned gslot = (unsigned)((gsub ^ swz(gkey)) * 16) + (unsigned)(hh * 5 * 128);
+  // Within a 128-byte group the 16-byte chunk c of key row r sits in slot c ^ (r & 7).  (The slot function of
+  // the other kernels' tiles also serves their transposing reads; with it this kernel's reads - 16 rows x 4
+  // chunks per instruction - take two LDS cycles where one is needed.)
+  const unsigned gslot = (unsigned)((gsub ^ (gkey & 7)) * 16) + (unsigned)(hh * 5 * 128);
   unsigned t_goff = 0, t_lb = 0;
   auto issue_prepare = [&](int n) {
     const int tile = tlist[n];
@@ -136,7 +139,7 @@ __device__ __forceinline__ void pds_body(
 #pragma unroll
     for (int par = 0; par < 2; par++) {
       const int row = 16 * kt + m;
-      boff[kt][par] = (unsigned)(row * 128 + (((4 * par + kg) ^ swz(row)) << 4));
+      boff[kt][par] = (unsigned)(row * 128 + (((4 * par + kg) ^ (row & 7)) << 4));
     }
   const float c2 = sm_scale * LOG2E;
 
