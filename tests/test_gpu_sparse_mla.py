@@ -114,6 +114,8 @@ def test_forward_slot_permutation_invariance(gpu):
     (64, 128, 64, 0, None, 0),
     (200, 128, 128, 40, 300, 3),
     (160, 64, 64, 0, None, 5),
+    (130, 32, 192, 5, 400, 7),           # two of pass A's eight 16-head waves hold real heads
+    (90, 96, 320, 0, None, 9),           # six of them; ten tiles per query
 ])
 def test_backward_against_oracle_and_deterministic(gpu, S, H, K, q_start, skv, seed):
     from loongforge_amd import ops
