@@ -247,16 +247,15 @@ __device__ __forceinline__ void pds_body(
 // ---------------------------------------------------------------------------------------------
 // dQ^T[d, head] += KV^T[d, key] . dS^T[key, head] per 32-key tile.  Both operands are LDS transpose
 // reads: of the gathered key tile (18 d-tiles) and of the tile's dS block copied verbatim from the
-// pass-A buffer.  Eight waves share the 72 accumulator tiles (18 d-tiles x 4 head groups): wave
-// (w, hh) = (wave % 4, wave / 4) owns d-tiles 4w .. 4w+3 for the head groups 2hh, 2hh+1, plus d-tile
-// 16 + w/2 for head group 2hh + w%2 - 9 tiles (144 accumulator registers) and 18 MFMAs per wave and
-// tile.  (The wave keeps its two head groups in the order hgs[0] = 2hh + w%2, hgs[1] = the other one,
-// so that the ninth tile always uses operand 0: a run-time choice between two MFMAs would make the
-// compiler copy the accumulator between registers right after an MFMA it cannot see into.)  At under 256 registers per lane two waves share a SIMD, so that while one of them is held
-// up issuing its part of the next tile's transfers (the address unit takes them at 64 B/clk for the
-// whole compute unit) the other one keeps the matrix pipe busy; with four waves of 288 accumulator
-// registers nothing filled that gap.  A key-tile operand read from LDS feeds two MFMAs: 112 KB of
-// LDS reads per tile, below the 147 KB the matrix pipe's time allows.
+// pass-A buffer.  Twelve waves share the 72 accumulator tiles (18 d-tiles x 4 head groups): wave
+// (dg, hp) = (wave % 6, wave / 6) owns d-tiles 3dg .. 3dg+2 for the head groups 2hp, 2hp+1: 6 tiles
+// (96 accumulator registers), 12 MFMAs and 20 transposing reads per wave and tile.  A wave issues one
+// LDS instruction per 40-odd cycles whatever its width, and a transposing read carries 8 bytes per
+// lane: with eight waves (9 tiles, 28 reads each) the reads of a wave took longer than the MFMAs of
+// the two waves of a SIMD together (1 200 against 1 152 cycles per tile).  Three waves per SIMD at
+// under 168 registers per lane issue them in two thirds of the time, and one wave's transfer issue and
+// waits run under the MFMAs of the other two.
+constexpr int DQ_THREADS = 768;
 template <int STAGES>
 __device__ __forceinline__ void dq_body(
     const __bf16* __restrict__ kv, const int* __restrict__ ids, const unsigned char* __restrict__ pds,
@@ -265,7 +264,7 @@ __device__ __forceinline__ void dq_body(
   constexpr int STAGE_BYTES = TILE_BYTES + PDS_KIND_BYTES;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int w = wave & 3, hh = wave >> 2;
+  const int dg = wave % 6, hp = wave / 6;
   const int r = lane & 31, g = lane >> 5;
   const int qi = q0 + ql;
   const int NT = K / BI;
@@ -273,140 +272,115 @@ __device__ __forceinline__ void dq_body(
   unsigned* tmask = (unsigned*)(idx_s + K);
   int* tlist = (int*)(tmask + NT);
   int* ntile_s = tlist + NT;
-  // (the helper is written for four waves; the other four repeat part of its work with equal results)
+  // (the helper is written for four waves; the others repeat part of its work with equal results)
   const int ntiles = stage_ids(ids, ql, K, Skv, q_start + qi, idx_s, tmask, tlist, ntile_s);
 
   const unsigned lds0 = (unsigned)(uintptr_t)smem;
-  const LaneOffsets lo = lane_offsets();
   // transposed read of the dS block: lane (blk, ii) points at key 16s + 8t + 4g + ii/4 and the 4 heads
   // 16*(blk&1) + 4*(ii&3) .. +3 of a head group.  In HBM the block is [head group][s'][g'][key][8 heads];
   // in LDS the 16-byte pieces of a head group are reordered to [key][s'][g'], so that the 16 pieces a
   // half-wave reads at once (4 keys x 4 head octets) are 256 consecutive bytes: no bank conflicts.
   unsigned ds_off[2][2];
+  // transposed read of the key tile for the wave's d-tiles 3dg + i (same formula as LaneOffsets::tr_off,
+  // with the parity of the d-tile known only at run time)
+  unsigned a_off[3][2][2];
   {
     const int blk = lane >> 4, ii = lane & 15, qq = ii & 3;
-#pragma unroll
-    for (int s = 0; s < 2; s++)
-#pragma unroll
-      for (int t = 0; t < 2; t++) {
-        const int key = 16 * s + 8 * t + 4 * g + (ii >> 2);
-        ds_off[s][t] = (unsigned)(TILE_BYTES + key * 64 + (blk & 1) * 32 + (qq & 1) * 16 + (qq >> 1) * 8);
-      }
-  }
-  // piece P of the LDS order comes from piece src_piece(P) of the HBM order; thread P moves piece P
-  auto src_piece = [](int P) { return (P >> 7) * 128 + ((P >> 1) & 1) * 64 + (P & 1) * 32 + ((P >> 2) & 31); };
-  const unsigned ds_src = (unsigned)src_piece(tid) * 16u;
-  // key-tile operand offsets of this wave's d-tiles: i = 0..3 -> d-tile 4*w + i, i = 4 -> 16 + w/2
-  const unsigned grp_main = (unsigned)(2 * w) * GRP_BYTES;             // (4w + i) >> 1 = 2w + (i >> 1)
-  const unsigned grp_last = (unsigned)(8 * GRP_BYTES);                 // (16 + w/2) >> 1 = 8
-  const int par_last = (w >> 1) & 1;
-  unsigned tr_last[2][2];
-  {
-    // same formula as LaneOffsets::tr_off, with the parity of the d-tile known only at run time
-    const int blk = lane >> 4, ii = lane & 15;
     const int cl = 2 * (blk & 1) + ((ii & 3) >> 1), half = ii & 1;
 #pragma unroll
     for (int s = 0; s < 2; s++)
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         const int key = 16 * s + 8 * t + 4 * g + (ii >> 2);
-        tr_last[s][t] = (unsigned)(key * 128 + (((4 * par_last + cl) ^ swz(key)) << 4) + half * 8) + grp_last;
+        ds_off[s][t] = (unsigned)(TILE_BYTES + key * 64 + (blk & 1) * 32 + (qq & 1) * 16 + (qq >> 1) * 8);
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+          const int dt = 3 * dg + i;
+          a_off[i][s][t] = (unsigned)((dt >> 1) * GRP_BYTES + key * 128 + (((4 * (dt & 1) + cl) ^ swz(key)) << 4) + half * 8);
+        }
       }
   }
-  // Transfers of a tile: the key rows as nine 128-byte groups per row, thread (key, sub) of either half of
-  // the workgroup moving 16 bytes of a group (waves 0-3 take groups 0-4, waves 4-7 groups 5-8), and the
-  // 8 KB dS block, 16 bytes per thread.
-  // transfers per wave and tile: 6 for waves 0-3, 5 for waves 4-7
-  auto issue = [&](int n) {
+  // Transfers of a tile: 44 of 1 KB each.  Transfer t < 36 is slot t % 4 (keys 8*slot .. +7, thread (key,
+  // sub) moving 16 bytes) of the 128-byte group t / 4 of the key rows; transfer 36 + b is 1 KB of the dS
+  // block, piece P of the LDS order coming from piece src_piece(P) of the HBM order.  Wave v takes
+  // transfers v, v + 12, v + 24 (groups v/4, v/4 + 3, v/4 + 6 of its slot v % 4) and, for v < 8, 36 + v.
+  auto src_piece = [](int P) { return (P >> 7) * 128 + ((P >> 1) & 1) * 64 + (P & 1) * 32 + ((P >> 2) & 31); };
+  const unsigned ds_src = (unsigned)src_piece((wave & 7) * 64 + lane) * 16u;
+  const int gkey = 8 * (wave & 3) + (lane >> 3), gsub = lane & 7;
+  const unsigned gslot = (unsigned)((gsub ^ swz(gkey)) * 16) + (unsigned)((wave >> 2) * 128);
+  unsigned t_goff = 0, t_lb = 0, t_lbd = 0;
+  const unsigned char* t_src = nullptr;
+  auto issue_prepare = [&](int n) {
     const int tile = tlist[n];
     const unsigned sb = lds0 + (unsigned)((n % STAGES) * STAGE_BYTES);
-    const int gkey = (tid & 255) >> 3, gsub = tid & 7;
     int kid = idx_s[tile * BI + gkey];
     kid = kid < 0 ? 0 : kid;
-    const unsigned goff = (unsigned)kid * (DQK * 2) + (unsigned)((gsub ^ swz(gkey)) * 16);
-    const unsigned lb = __builtin_amdgcn_readfirstlane(sb + (unsigned)(w * 1024));
-    if (hh == 0) {
-#pragma unroll
-      for (int grp = 0; grp < 5; grp++) dma16(lb + grp * GRP_BYTES, goff + grp * 128, kv);
-    } else {
-#pragma unroll
-      for (int grp = 5; grp < 9; grp++) dma16(lb + grp * GRP_BYTES, goff + grp * 128, kv);
-    }
-    const unsigned lbd = __builtin_amdgcn_readfirstlane(sb + (unsigned)(TILE_BYTES + wave * 1024));
-    const unsigned char* src = uniform_ptr(pds + ((size_t)ql * NT + tile) * PDS_TILE_BYTES);     // dS half
-    dma16(lbd, ds_src, src);
+    t_goff = (unsigned)kid * (DQK * 2) + gslot;
+    t_lb = __builtin_amdgcn_readfirstlane(sb + (unsigned)((wave & 3) * 1024 + (wave >> 2) * GRP_BYTES));
+    t_lbd = __builtin_amdgcn_readfirstlane(sb + (unsigned)(TILE_BYTES + (wave & 7) * 1024));
+    t_src = uniform_ptr(pds + ((size_t)ql * NT + tile) * PDS_TILE_BYTES);     // dS half
+  };
+  // step 0 .. 2: the wave's three groups of the key rows; step 3: its part of the dS block (waves 0-7)
+  auto issue_step = [&](int j) {
+    if (j < 3) dma16(t_lb + 3 * j * GRP_BYTES, t_goff + 3 * j * 128, kv);
+    else if (wave < 8) dma16(t_lbd, ds_src, t_src);
   };
 
-  const int hg0 = 2 * hh + (w & 1), hg1 = 2 * hh + 1 - (w & 1);       // the wave's head groups, in its operand order
-  f32x16 acc[9];      // u < 8: d-tile 4w + u/2, head group hg0 (u even) or hg1 (u odd); u = 8: d-tile 16 + w/2, head group hg0
+  const int hg0 = 2 * hp, hg1 = 2 * hp + 1;
+  f32x16 acc[6];      // u = 2 * i + j: d-tile 3dg + i, head group 2hp + j
 #pragma unroll
-  for (int u = 0; u < 9; u++) {
+  for (int u = 0; u < 6; u++)
 #pragma unroll
     for (int e = 0; e < 16; e++) acc[u][e] = 0.f;
-    if (u < 8) asm volatile("" : "+a"(acc[u])); else asm volatile("" : "+v"(acc[u]));
-  }
   typedef short i16x8 __attribute__((ext_vector_type(8)));
   auto tr_pair = [&](const unsigned char* p0, const unsigned char* p1) {
     const i16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, p0));
     const i16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(i16x4, p1));
     return __builtin_bit_cast(bf16x8, (i16x8)__builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
   };
-  for (int n = 0; n < STAGES - 1 && n < ntiles; n++) issue(n);
+  for (int n = 0; n < STAGES - 1 && n < ntiles; n++) {
+    issue_prepare(n);
+#pragma unroll
+    for (int j = 0; j < 4; j++) issue_step(j);
+  }
   for (int n = 0; n < ntiles; n++) {
     static_assert(STAGES == 3, "one tile of transfers in flight behind the awaited one");
-    if (n + 1 < ntiles) { if (hh) { DSA_WAIT_VMCNT(5); } else { DSA_WAIT_VMCNT(6); } } else { DSA_WAIT_VMCNT(0); }
+    // transfers per wave and tile: 4 for waves 0-7, 3 for waves 8-11
+    if (n + 1 < ntiles) { if (wave < 8) { DSA_WAIT_VMCNT(4); } else { DSA_WAIT_VMCNT(3); } } else { DSA_WAIT_VMCNT(0); }
     __syncthreads();
-    // The two waves of a SIMD (w, 0) and (w, 1) issue their transfers at different times - here and after
-    // the second d-tile - so that each does so while the other one feeds the matrix pipe.
-    if (hh == 0 && n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
+    const bool more = n + STAGES - 1 < ntiles;
+    if (more) { issue_prepare(n + STAGES - 1); issue_step(3); }
     const unsigned char* tb = smem + (n % STAGES) * STAGE_BYTES;
-    // the four dS operands of the wave's two head groups: [hg0 or hg1][k-step]
-    bf16x8 bds[2][2];
+    // key-tile operands one d-tile ahead, the four dS operands of the wave's two head groups: [hg0 or hg1][k-step]
+    bf16x8 a[2][2], bds[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; s++) a[0][s] = tr_pair(tb + a_off[0][s][0], tb + a_off[0][s][1]);
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int s = 0; s < 2; s++)
         bds[j][s] = tr_pair(tb + (j ? hg1 : hg0) * 2048 + ds_off[s][0], tb + (j ? hg1 : hg0) * 2048 + ds_off[s][1]);
-    // key-tile operands, one d-tile ahead
-    bf16x8 a[2][2];
-#pragma unroll
-    for (int s = 0; s < 2; s++)
-      a[0][s] = tr_pair(tb + grp_main + lo.tr_off[s][0][0], tb + grp_main + lo.tr_off[s][1][0]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < 5; i++) {
-      if (i + 1 < 5) {
+    for (int i = 0; i < 3; i++) {
+      if (i + 1 < 3) {
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-          if (i + 1 < 4)
-            a[(i + 1) & 1][s] = tr_pair(tb + grp_main + ((i + 1) >> 1) * GRP_BYTES + lo.tr_off[s][0][(i + 1) & 1],
-                                        tb + grp_main + ((i + 1) >> 1) * GRP_BYTES + lo.tr_off[s][1][(i + 1) & 1]);
-          else
-            a[(i + 1) & 1][s] = tr_pair(tb + tr_last[s][0], tb + tr_last[s][1]);
-        }
+        for (int s = 0; s < 2; s++) a[(i + 1) & 1][s] = tr_pair(tb + a_off[i + 1][s][0], tb + a_off[i + 1][s][1]);
       }
 #pragma unroll
-      for (int s = 0; s < 2; s++) {
-        if (i < 4) {
+      for (int s = 0; s < 2; s++)
 #pragma unroll
-          for (int j = 0; j < 2; j++) mfma_a_vv(acc[2 * i + j], a[i & 1][s], bds[j][s]);
-        } else {
-          mfma_v_vv(acc[8], a[i & 1][s], bds[0][s]);
-        }
-      }
+        for (int j = 0; j < 2; j++)
+          acc[2 * i + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i & 1][s], bds[j][s], acc[2 * i + j], 0, 0, 0);
+      if (more) issue_step(i);
       __builtin_amdgcn_sched_barrier(0);
-      if (i == 1) {
-        if (hh == 1 && n + STAGES - 1 < ntiles) issue(n + STAGES - 1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
     }
   }
   // ---- write dQ: accumulator e of a lane is d = 32*dt + 8*(e/4) + 4*g + (e%4), head = 32*hg + r ----
   const bool poison = *dup_flag != 0;          // a query row with a repeated id: NaN instead of a sum that misses a term
 #pragma unroll
-  for (int u = 0; u < 9; u++) {
-    if (u < 8) mfma_done_a(acc[u]); else mfma_done_v(acc[u]);
-    const int dt = u < 8 ? 4 * w + (u >> 1) : 16 + (w >> 1);
+  for (int u = 0; u < 6; u++) {
+    const int dt = 3 * dg + (u >> 1);
     const int hg = (u & 1) ? hg1 : hg0;
     const int h = hg * 32 + r;
     if (h < H) {                               // the same for all lanes of a wave (H is a multiple of 32)
@@ -659,7 +633,7 @@ __device__ __forceinline__ void dkv_body(
 // ---------------------------------------------------------------------------------------------
 // pass D: dKV[key] = sum of that key's rows, ascending query order
 // ---------------------------------------------------------------------------------------------
-// One key per workgroup of 512 threads: 72 column chunks of 8 elements x 7 row groups (row r of the
+// One key per workgroup (504 of its threads): 72 column chunks of 8 elements x 7 row groups (row r of the
 // segment goes to group r % 7); the seven partial sums are combined in a fixed order, so the result
 // depends only on the segment, never on scheduling.  Pure streaming reads of 1152-byte rows, RED_FLIGHT
 // of them in flight per thread.
@@ -703,7 +677,7 @@ __device__ __forceinline__ void reduce_body(const unsigned char* __restrict__ ro
     for (int e = 0; e < 8; e++) part[grp * DQK + ch * 8 + e] = acc[e];
   }
   __syncthreads();
-  for (int d = tid; d < DQK; d += 512) {
+  for (int d = tid; d < DQK; d += (int)blockDim.x) {
     float s = part[d];
 #pragma unroll
     for (int gq = 1; gq < RED_GROUPS; gq++) s += part[gq * DQK + d];
@@ -756,7 +730,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(
   else dkv_body<4>(q, dout, ids, pds, dst, rows, q0, ql, H, Skv, K, q_start, dummy_row, smem);
 }
 
-__global__ __launch_bounds__(512, 1) void bwd_dq_reduce_kernel(
+__global__ __launch_bounds__(DQ_THREADS, 1) void bwd_dq_reduce_kernel(
     const __bf16* __restrict__ kv, const int* __restrict__ ids, const unsigned char* __restrict__ pds,
     __bf16* __restrict__ dq, int q0, int cnt, int H, int Skv, int K, int q_start, const int* __restrict__ dup_flag,
     const unsigned char* __restrict__ rows, const int* __restrict__ start, float* __restrict__ dkv_acc, int n_keys,
@@ -902,7 +876,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV rows)");
     DSA_MARK(3);
     // Pass B of every query beside pass D of every key.
-    bwd_dq_reduce_kernel<<<dim3(cnt + Skv), dim3(512), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv,
+    bwd_dq_reduce_kernel<<<dim3(cnt + Skv), dim3(DQ_THREADS), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv,
                                                                    K, q_start, dup_flag, rows, start, acc, Skv, first ? 0 : 1);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ | dKV reduce)");
     DSA_MARK(4);
