@@ -352,3 +352,40 @@ def test_attn_dist_from_q_kv_lse_with_sink_is_the_softmax_over_the_slots(gpu):
     got = ops.attn_dist_qk(q, kv, ids, lse, 0, inp.sm_scale, 128, attn_sink=sink.to(gpu))
     _, _, rp = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, 0, inp.sm_scale, 512)
     assert (got.cpu() - O.attn_dist(rp, inp.sm_scale)).abs().max().item() <= 5e-5
+
+
+def test_random_shapes_forward_backward_distribution(gpu):
+    """Sixteen seeded random shapes (32 - 128 heads, 1 - 8 tiles per query, chunk offsets, longer key arrays, slot
+    lists with holes): forward, backward by the parity rule, bit-equal reruns, recomputed attention distribution."""
+    import random
+
+    from loongforge_amd import ops
+
+    rng = random.Random(1234)
+    for case in range(16):
+        H = rng.choice([32, 64, 96, 128])
+        K = 64 * rng.randint(1, 8)
+        S = rng.randint(1, 160)
+        q_start = rng.choice([0, 0, rng.randint(1, 300)])
+        skv = q_start + S + rng.choice([0, 0, rng.randint(1, 100)])
+        seed = rng.randint(0, 10 ** 6)
+        name = "case %d S=%d H=%d K=%d q_start=%d skv=%d seed=%d" % (case, S, H, K, q_start, skv, seed)
+        print(name, flush=True)
+        inp = O.make_mla_inputs(S, H, K, seed=seed, skv=skv, q_start=q_start)
+        if rng.random() < 0.3:
+            holes = torch.rand(inp.idx.shape, generator=torch.Generator().manual_seed(seed)) < 0.3
+            inp.idx[holes] = -1
+        q, kv, idx, do = inp.q.to(gpu), inp.kv.to(gpu), inp.idx.to(gpu), inp.dout.to(gpu)
+        out, lse, _ = ops.sparse_mla_fwd(q, kv, idx, q_start, inp.sm_scale)
+        ro, rl, _ = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, q_start, inp.sm_scale)
+        assert_close(out, ro, name + " out", atol=2e-2, rtol=0)
+        fin = torch.isfinite(rl)
+        assert torch.equal(torch.isfinite(lse.cpu()), fin), name
+        assert_close(lse.cpu()[fin], rl[fin], name + " lse", atol=1e-3, rtol=0)
+        dq, dkv = ops.sparse_mla_bwd(q, kv, out, do, idx, lse, q_start, inp.sm_scale)
+        dq2, dkv2 = ops.sparse_mla_bwd(q, kv, out, do, idx, lse, q_start, inp.sm_scale)
+        assert torch.equal(dq, dq2) and torch.equal(dkv, dkv2), name
+        assert_mla_grads(dq, dkv, inp.q, inp.kv, inp.idx, inp.dout, q_start, inp.sm_scale, name=name, out=out, lse=lse)
+        target = ops.attn_dist_qk(q, kv, idx, lse, q_start, inp.sm_scale, H)
+        ref = O.attn_dist_from_lse(inp.q, inp.kv, inp.idx, lse.cpu(), q_start, inp.sm_scale, H)
+        assert_close(target, ref, name + " attn_dist", atol=1e-3, rtol=1e-2)
