@@ -81,3 +81,15 @@ def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libdsa_hip.so"))
     with pytest.raises(_lib.DsaError, match="missing"):
         _lib.load()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU; asked for more it says so and exits without touching a device."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                         timeout=120)
+    assert res.returncode != 0
+    assert "one GPU" in (res.stdout + res.stderr)
