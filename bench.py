@@ -454,14 +454,24 @@ def main():
             traffic_note = "rocprofv3 FETCH_SIZE + WRITE_SIZE of profiles/traffic.json, taken with these kernel sources"
         else:
             traffic_note = "profiles/traffic.json was taken with other kernel sources: dropped"
-    roofline = {"kernel": name, "bound": "mfma", "achieved": round(f_dom / (t_dom * 1e-3) / 1e12, 1),
-                "peak": PEAK_BF16, "unit": "TFLOP/s", "traffic": traffic, "traffic_note": traffic_note}
+    # The roof that binds that launch is the one it sits closer to: HBM (8 TB/s) when its bytes over its time are
+    # the larger fraction of peak, else the bf16 MFMA peak; the other figure stays beside it.
+    gbps_dom = b_dom / (t_dom * 1e-3) / 1e9
+    tflops_dom = f_dom / (t_dom * 1e-3) / 1e12
+    hbm_bound = gbps_dom / 8000.0 > tflops_dom / PEAK_BF16
+    if hbm_bound:
+        roofline = {"kernel": name, "bound": "hbm", "achieved": round(gbps_dom, 1), "peak": 8000.0, "unit": "GB/s"}
+        roofline["mfma"] = {"achieved": round(tflops_dom, 1), "peak": PEAK_BF16, "unit": "TFLOP/s",
+                            "frac": round(tflops_dom / PEAK_BF16, 4)}
+    else:
+        roofline = {"kernel": name, "bound": "mfma", "achieved": round(tflops_dom, 1), "peak": PEAK_BF16, "unit": "TFLOP/s"}
+        roofline["hbm"] = {"achieved": round(gbps_dom, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(gbps_dom / 8000.0, 4)}
+    roofline["traffic"] = traffic
+    roofline["traffic_note"] = traffic_note
     roofline["frac"] = round(roofline["achieved"] / roofline["peak"], 4)
     roofline["avg_launch_ms"] = round(t_dom, 3)
     roofline["algorithmic_flops"] = f_dom
     roofline["design_hbm_bytes"] = b_dom          # what this build's passes move in that launch, intermediates included
-    roofline["design_hbm_gbps"] = round(b_dom / (t_dom * 1e-3) / 1e9, 1)
-    roofline["design_hbm_frac_of_8tbps"] = round(b_dom / (t_dom * 1e-3) / 8e12, 4)
     # the whole backward: bytes an ideal implementation moves (Q, dO, O in; dQ, dKV out) against this design's
     ideal_bwd = b_q + b_do + b_o + b_dq + b_dkv
     design_bwd = sum(pass_bytes)

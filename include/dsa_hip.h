@@ -202,8 +202,14 @@ int dsa_sparse_mla_fwd_ex(const void* q, const void* kv, const int32_t* ids, int
  * sparse_mla_bwd_interface as called at dsa_fused_kernels.py:2086-2110
  * (math: loongforge/models/common/experimental_attention_variant/sparse_mla_bwd.py:292-356).
  *   dout [S, H, 512] bf16   dq [S, H, 576] bf16   dkv [Skv, 576] bf16
+ * Workspace: dsa_sparse_mla_bwd_workspace_bytes is the largest size the call can use - all queries in one
+ * sweep (26 GiB at S = Skv = 8192, K = 2048; 105 GiB at 32768 tokens).  Any size from
+ * dsa_sparse_mla_bwd_workspace_bytes_min on is accepted: with less than the full size the queries are walked in
+ * chunks (the largest of S, S/2, S/4, ... that fits, at least 64), a few per cent slower per extra chunk; the
+ * chunking follows from the sizes alone, and dKV is bit-reproducible for a given workspace size.
  */
 size_t dsa_sparse_mla_bwd_workspace_bytes(int S, int H, int Skv, int K);
+size_t dsa_sparse_mla_bwd_workspace_bytes_min(int S, int H, int Skv, int K);
 int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out, const void* dout,
                        const int32_t* ids, const float* lse, int S, int H, int Skv, int K,
                        int q_start, float sm_scale, int d_v, void* dq, void* dkv,

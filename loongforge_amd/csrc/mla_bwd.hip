@@ -756,6 +756,13 @@ __global__ void cast_bf16_kernel(const float* __restrict__ src, unsigned short* 
     dstp[e] = poison ? (unsigned short)0x7fc0 : f32_to_bf16_bits(src[e]);
 }
 
+// dQ of the chunks that ran before the flag was raised still holds sums: NaN everywhere in that case
+__global__ void poison_bf16_kernel(unsigned short* __restrict__ p, size_t n, const int* __restrict__ dup_flag) {
+  if (*dup_flag == 0) return;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x)
+    p[e] = (unsigned short)0x7fc0;
+}
+
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
@@ -806,6 +813,12 @@ extern "C" size_t dsa_sparse_mla_bwd_workspace_bytes(int S, int H, int Skv, int 
   (void)H;
   if (S <= 0 || Skv <= 0 || K <= 0) return 0;
   return make_plan(S, Skv, K, DEFAULT_BUDGET).total;
+}
+
+extern "C" size_t dsa_sparse_mla_bwd_workspace_bytes_min(int S, int H, int Skv, int K) {
+  (void)H;
+  if (S <= 0 || Skv <= 0 || K <= 0) return 0;
+  return layout_plan(S < 64 ? S : 64, Skv, K).total;
 }
 
 static int bwd_impl(const void* q, const void* kv, const void* out, const void* dout, const int32_t* ids,
@@ -897,6 +910,8 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     order::zero_u32_kernel<<<dim3(256), dim3(256), 0, st>>>((unsigned*)acc, (size_t)Skv * DQK);
   }
   cast_bf16_kernel<<<dim3(2048), dim3(256), 0, st>>>(acc, (unsigned short*)dkv, (size_t)Skv * DQK, dup_flag);
+  if (S > p.chunk)      // more than one chunk: the flag may have come up after earlier chunks wrote their dQ
+    poison_bf16_kernel<<<dim3(2048), dim3(256), 0, st>>>((unsigned short*)dq, (size_t)S * H * DQK, dup_flag);
   DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(cast)");
   (void)NT;
   if (pass_ms) for (int i = 0; i < 5; i++) hipEventDestroy(ev[i]);

@@ -447,15 +447,18 @@ def sparse_mla_fwd(q, kv, ids, q_start: int = 0, sm_scale: Optional[float] = Non
 
 
 _BWD_WS = {}      # device index -> workspace kept between calls
+BWD_MAX_SLOTS = 2048      # slots per query the backward kernels take in one call
+ATTN_DIST_QK_MAX_SLOTS = 4096
 
 
 def _bwd_workspace(full_bytes: int, device):
     """Workspace of the sparse-MLA backward: ``full_bytes`` lets it take all queries in one sweep (26 GiB at 8k
-    tokens, top-k 2048; 105 GiB at 32k); given less, the library walks the queries in chunks (about 10 % slower at
-    32k tokens in three chunks).  The size is capped by ``DSA_BWD_WORKSPACE_GIB`` (default 48) and by 80 % of the
-    memory that is free, and the buffer is kept per device
-    and reused by later calls (calls that overlap on one device - other streams - must not share it: set
-    ``DSA_BWD_WORKSPACE_CACHE=0``).  Nothing is kept while a HIP graph is being captured."""
+    tokens, top-k 2048; 105 GiB at 32k); given less, the library walks the queries in chunks.  The size handed to
+    the library - and with it the chunking, on which the last bits of dKV depend - follows from the shapes and
+    from ``DSA_BWD_WORKSPACE_GIB`` (default 48) alone, never from what happens to be free or from earlier calls.
+    The buffer is kept per device and reused by later calls (held until :func:`release_bwd_workspace`; calls that
+    overlap on one device - other streams - must not share it: set ``DSA_BWD_WORKSPACE_CACHE=0``).  Nothing is
+    kept while a HIP graph is being captured."""
     want = max(int(full_bytes), 256)
     cap = os.environ.get("DSA_BWD_WORKSPACE_GIB", "48")
     want = min(want, max(int(float(cap) * 2 ** 30), 256))
@@ -463,17 +466,25 @@ def _bwd_workspace(full_bytes: int, device):
     kept = _BWD_WS.get(idx)
     if kept is not None and kept.numel() >= want:
         return kept, want
-    free, _ = torch.cuda.mem_get_info(idx)
-    free += kept.numel() if kept is not None else 0
-    want = min(want, max(int(free * 0.8), 256))
-    if kept is not None and kept.numel() >= want:
-        return kept, want
     _BWD_WS.pop(idx, None)
     del kept
-    ws = torch.empty(want, dtype=torch.uint8, device=device)
+    try:
+        ws = torch.empty(want, dtype=torch.uint8, device=device)
+    except torch.OutOfMemoryError as e:
+        raise RuntimeError("sparse_mla_bwd: cannot allocate its %.1f GiB workspace; lower DSA_BWD_WORKSPACE_GIB "
+                           "(the library then walks the queries in more chunks)" % (want / 2 ** 30)) from e
     if os.environ.get("DSA_BWD_WORKSPACE_CACHE", "1") != "0" and not torch.cuda.is_current_stream_capturing():
         _BWD_WS[idx] = ws
     return ws, want
+
+
+def release_bwd_workspace(device=None):
+    """Drops the backward workspace kept for ``device`` (all devices if None)."""
+    if device is None:
+        _BWD_WS.clear()
+    else:
+        d = torch.device(device)
+        _BWD_WS.pop(d.index if d.index is not None else torch.cuda.current_device(), None)
 
 
 @torch.library.custom_op("dsa::sparse_mla_bwd", mutates_args=())
@@ -505,10 +516,25 @@ def _(q, kv, out, dout, ids, lse, q_start, sm_scale, d_v):
 
 
 def sparse_mla_bwd(q, kv, out, dout, ids, lse, q_start: int = 0, sm_scale: Optional[float] = None, d_v: int = 512):
-    """(dq, dkv) in bf16; dkv is accumulated in a fixed order (bit-reproducible)."""
+    """(dq, dkv) in bf16; dkv is accumulated in a fixed order (bit-reproducible).
+
+    The kernels take up to 2048 slots per query.  Longer lists are walked 2048 slots at a time: with the
+    softmax statistics (``lse``) and ``out`` of the whole list given, the gradients are sums over the slots, so the
+    parts add up (in fp32 here; an id that a query holds in two different parts is not detected)."""
     if sm_scale is None:
         sm_scale = q.shape[-1] ** -0.5
-    return _mla_bwd_op(q, kv, out, dout, ids, lse, int(q_start), float(sm_scale), int(d_v))
+    K = ids.shape[1]
+    if K <= BWD_MAX_SLOTS:
+        return _mla_bwd_op(q, kv, out, dout, ids, lse, int(q_start), float(sm_scale), int(d_v))
+    dq32 = dkv32 = None
+    for k0 in range(0, K, BWD_MAX_SLOTS):
+        part = ids[:, k0:k0 + BWD_MAX_SLOTS]
+        if part.shape[1] % 64:
+            part = torch.nn.functional.pad(part, (0, 64 - part.shape[1] % 64), value=-1)
+        dq, dkv = _mla_bwd_op(q, kv, out, dout, part.contiguous(), lse, int(q_start), float(sm_scale), int(d_v))
+        dq32 = dq.float() if dq32 is None else dq32.add_(dq)
+        dkv32 = dkv.float() if dkv32 is None else dkv32.add_(dkv)
+    return dq32.to(torch.bfloat16), dkv32.to(torch.bfloat16)
 
 
 @torch.library.custom_op("dsa::attn_dist", mutates_args=())
@@ -574,7 +600,19 @@ def attn_dist_qk(q, kv, ids, lse, q_start: int, sm_scale: float, heads_in_mean: 
     ``lse + log(1 - exp(sink - lse))``, which is what the kernel is given then."""
     if attn_sink is not None:
         lse = lse + torch.log1p(-torch.exp(attn_sink.to(lse.dtype).view(1, -1) - lse).clamp(max=1.0 - 1e-7))
-    return _attn_dist_qk_op(q, kv, ids, lse, int(q_start), float(sm_scale), int(heads_in_mean or q.shape[1]))
+    hm = int(heads_in_mean or q.shape[1])
+    K = ids.shape[1]
+    if K <= ATTN_DIST_QK_MAX_SLOTS:
+        return _attn_dist_qk_op(q, kv, ids, lse, int(q_start), float(sm_scale), hm)
+    # the kernel takes up to 4096 slots; with lse given every slot's value stands alone, so longer lists go in parts
+    parts = []
+    for k0 in range(0, K, ATTN_DIST_QK_MAX_SLOTS):
+        part = ids[:, k0:k0 + ATTN_DIST_QK_MAX_SLOTS]
+        n = part.shape[1]
+        if n % 64:
+            part = torch.nn.functional.pad(part, (0, 64 - n % 64), value=-1)
+        parts.append(_attn_dist_qk_op(q, kv, part.contiguous(), lse, int(q_start), float(sm_scale), hm)[:, :n])
+    return torch.cat(parts, dim=1)
 
 
 # --------------------------------------------------------------------------------------------

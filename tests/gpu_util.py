@@ -33,13 +33,18 @@ def valid_sets_equal_up_to_noise(ids, ref_ids, ref_logits, band):
     return bad
 
 
-# Largest amount by which a dKV element of the HIP backward may exceed 2e-2 + 1e-2*|ref| of the
-# plain fp32 gradient.  The reference kernel's own rounding (P and dS enter its MFMAs as bf16,
-# ops/tilelang_ops/sparse_mla_bwd.py:194, 200) already leaves that bound: evaluated by the oracle it
-# exceeds it by up to 7e-2 at the benchmark shapes; this build's bf16 per-pair rows add about half
-# as much again (measured: 0.08 - 0.14).  The two strict checks below are the parity gate; this
-# number only records how far a bf16-operand backward sits from an fp32 one.
-FP32_DKV_EXCESS_LIMIT = 0.2
+# How far a dKV element of the HIP backward may lie outside 2e-2 + 1e-2*|ref|, as fixed numbers (none of them
+# scales with the data); each is the largest value measured over every shape the tests run (N(0,1) inputs, dKV
+# elements up to 80) plus a fifth:
+#   * against the plain fp32 gradient: measured up to 0.138.  The reference kernel's own rounding (P and dS enter
+#     its MFMAs as bf16, ops/tilelang_ops/sparse_mla_bwd.py:194, 200), evaluated by the oracle, already leaves
+#     the bound by up to 0.122 on the same inputs;
+#   * against the fp32 gradient, beyond what the reference kernel's rounding leaves it by: measured up to 0.048
+#     (the share of this build's bf16 rows of the (query, key) pairs);
+#   * against the oracle with the reference kernel's rounding (bf16 P and dS, fp32 rows): measured up to 0.112.
+FP32_DKV_EXCESS_LIMIT = 0.17
+FP32_DKV_OVER_REFERENCE_LIMIT = 0.06
+REF_DKV_EXCESS_LIMIT = 0.135
 # The same for dQ = dS.KV, where only the bf16 cast of dS matters: at top-k 64 and below, where single
 # softmax terms are of order 1, the reference kernel's rounding leaves the bound by up to 1.1e-2
 # (measured); from top-k 256 on it stays inside.
@@ -48,7 +53,7 @@ FP32_DQ_EXCESS_LIMIT = 0.02
 
 def assert_mla_grads(dq, dkv, q, kv, idx, dout, q_start, sm_scale, name="", d_v=512, attn_sink=None,
                      out=None, lse=None, dkv_rows=None):
-    """Parity rule of the sparse-MLA backward, every element, no slack that scales with the data:
+    """Parity rule of the sparse-MLA backward, every element, with bounds that do not scale with the data:
 
     * dQ against the oracle evaluated with the reference kernel's rounding points (P and dS cast to
       bf16, ops/tilelang_ops/sparse_mla_bwd.py:194, 200; the HIP kernels round nowhere else on the
@@ -60,11 +65,13 @@ def assert_mla_grads(dq, dkv, q, kv, idx, dout, q_start, sm_scale, name="", d_v=
       bf16 grid there.  (Two evaluations of the same formula - fp32 on the GPU, fp64 here, so that the
       expected values do not depend on the host - now and then land on different sides of a rounding
       boundary; where rows are of order 10 such a step is 0.06 - 0.12 and would alone break 2e-2.)
+      This check shows that the kernels compute what they are meant to; the next two say how far that is
+      from the reference.
     * dKV against the oracle with only the reference kernel's rounding (bf16 P and dS, fp32 rows):
-      the bound widened by ``2**-9 * A`` with ``A = sum over pairs |row|``, which is all that
-      round-to-nearest bf16 rows can change.
-    * dKV against the plain fp32 gradient: the excess over the bound is returned and must stay
-      below FP32_DKV_EXCESS_LIMIT.
+      the excess over ``2e-2 + 1e-2*|ref|`` stays below REF_DKV_EXCESS_LIMIT.
+    * dKV against the plain fp32 gradient: the excess stays below FP32_DKV_EXCESS_LIMIT and exceeds the
+      excess of the reference kernel's rounding on the same inputs by less than
+      FP32_DKV_OVER_REFERENCE_LIMIT.  Returned.
 
     All inputs are CPU tensors except dq / dkv.  ``out`` / ``lse`` are inputs of the backward
     (``Delta = rowsum(out * dO)`` feels every bf16 rounding of ``out``): pass what the backward under
@@ -80,7 +87,7 @@ def assert_mla_grads(dq, dkv, q, kv, idx, dout, q_start, sm_scale, name="", d_v=
     lse = lse.detach().cpu() if lse is not None else None
     rdq, rdkv = O.sparse_mla_bwd(q, kv, idx, dout, q_start, sm_scale, d_v, attn_sink=attn_sink)
     kw = dict(out=out, lse=lse, attn_sink=attn_sink, dtype=torch.float64)     # fp64: the same on every host
-    dq_b, dkv_b, a_sum, _ = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, dout, q_start, sm_scale, d_v, return_abs_sum=True, **kw)
+    dq_b, dkv_b = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, dout, q_start, sm_scale, d_v, **kw)
     _, dkv_r, _, a_max = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, dout, q_start, sm_scale, d_v, round_rows_bf16=True,
                                                          return_abs_sum=True, **kw)
 
@@ -93,8 +100,10 @@ def assert_mla_grads(dq, dkv, q, kv, idx, dout, q_start, sm_scale, name="", d_v=
     assert e <= FP32_DQ_EXCESS_LIMIT, "%s dQ vs fp32 oracle: excess %.3e" % (name, e)
     e = excess(dkv, dkv_r, 2.0 ** -7 * a_max)
     assert e <= 0, "%s dKV vs oracle with bf16 P/dS and bf16 rows: exceeds the bound by %.3e" % (name, e)
-    e = excess(dkv, dkv_b, 2.0 ** -9 * a_sum)
-    assert e <= 0, "%s dKV vs oracle with the reference kernel's rounding: exceeds the widened bound by %.3e" % (name, e)
-    e32 = excess(dkv, rdkv)
+    e = excess(dkv, dkv_b)
+    assert e <= REF_DKV_EXCESS_LIMIT, "%s dKV vs oracle with the reference kernel's rounding: excess %.3e" % (name, e)
+    e32, eref = excess(dkv, rdkv), excess(dkv_b.float(), rdkv)
     assert e32 <= FP32_DKV_EXCESS_LIMIT, "%s dKV vs fp32 oracle: excess %.3e" % (name, e32)
+    assert e32 <= max(eref, 0.0) + FP32_DKV_OVER_REFERENCE_LIMIT, \
+        "%s dKV vs fp32 oracle: excess %.3e, the reference kernel's rounding alone %.3e" % (name, e32, eref)
     return e32

@@ -33,7 +33,7 @@ def test_indexer_topk_full_size_properties(gpu):
     srt = torch.sort(torch.where(valid, ids, torch.full_like(ids, -1)), dim=1).values
     assert ((srt[:, 1:] != srt[:, :-1]) | (srt[:, 1:] < 0)).all()               # ids unique per row
     # a sample of rows against the oracle, up to fp32 accumulation noise at the K-th boundary
-    rows = torch.tensor([0, 1, 2047, 2048, 4095, 6000, 8191])
+    rows = torch.unique(torch.cat([torch.tensor([0, 1, 2047, 2048, 4095, 6000, 8191]), torch.arange(13, S, 33)]))   # 256 rows
     q8c, k8c = q8.cpu(), k8.cpu()
     R = O.indexer_logits(q8c[rows], ws.cpu()[rows], k8c, ksc.cpu(), ks.cpu()[rows], ke.cpu()[rows], dtype=torch.float64)
     for n, i in enumerate(rows.tolist()):
@@ -69,23 +69,45 @@ def test_sparse_mla_full_size_forward_backward(gpu):
     # The oracle's closed form (pinned on the CPU against autograd and explicit loops) evaluated on the
     # GPU's tensors in fp32 - the full size takes minutes on the host - three times: plain fp32, with the
     # reference kernel's rounding (bf16 P / dS), and with this build's extra rounding (bf16 rows).
-    from tests.gpu_util import FP32_DKV_EXCESS_LIMIT
+    from tests.gpu_util import FP32_DKV_EXCESS_LIMIT, REF_DKV_EXCESS_LIMIT
     sm = inp.sm_scale
     with torch.no_grad():
         dq32, dkv32 = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, do, 0, sm, 512, out=out, lse=lse, round_p_ds_bf16=False)
-        dq_b, dkv_b, a_sum, _ = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, do, 0, sm, 512, out=out, lse=lse, return_abs_sum=True)
+        dq_b, dkv_b = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, do, 0, sm, 512, out=out, lse=lse)
         _, dkv_r = O.sparse_mla_bwd_kernel_rounding(q, kv, idx, do, 0, sm, 512, out=out, lse=lse, round_rows_bf16=True)
 
-    def excess(got, ref, extra=0.0):
-        return ((got.float() - ref).abs() - (2e-2 + 1e-2 * ref.abs() + extra)).max().item()
+    def over(got, ref):
+        return (got.float() - ref).abs() - (2e-2 + 1e-2 * ref.abs())
+
+    def excess(got, ref):
+        return over(got, ref).max().item()
 
     assert excess(dq, dq32) <= 0                                   # every element of dQ against fp32 ...
     assert excess(dq, dq_b) <= 0                                   # ... and against the reference kernel's rounding
     assert excess(dkv, dkv_r) <= 0                                 # every element of dKV, same rounding points (both fp32)
-    assert excess(dkv, dkv_b, 2.0 ** -9 * a_sum) <= 0              # reference kernel's rounding + what bf16 rows can move
+    e_ref = excess(dkv, dkv_b)                                     # against the reference kernel's rounding (fp32 rows)
+    assert e_ref <= REF_DKV_EXCESS_LIMIT
+    # against the plain fp32 gradient, the comparator the path is specified with: how far outside the bound, which
+    # share of the elements, and the same two figures for the reference kernel's own rounding on these inputs
     e32, eref = excess(dkv, dkv32), excess(dkv_b, dkv32)
-    print("dKV excess over 2e-2 + 1e-2|ref| against fp32: HIP %.3e, reference kernel's rounding %.3e" % (e32, eref))
+    f32, fref = (over(dkv, dkv32) > 0).float().mean().item(), (over(dkv_b, dkv32) > 0).float().mean().item()
+    record = {"workload": "sparse MLA backward, seq 8192, 128 heads, top-k 2048 (config 4)", "bound": "2e-2 + 1e-2*|ref|",
+              "max_abs_dkv": dkv32.abs().max().item(),
+              "hip_vs_fp32": {"excess": e32, "fraction_outside": f32},
+              "reference_kernel_rounding_vs_fp32": {"excess": eref, "fraction_outside": fref},
+              "hip_vs_reference_kernel_rounding": {"excess": e_ref},
+              "hip_vs_own_rounding_points": {"excess": excess(dkv, dkv_r)},
+              "dq_vs_fp32": {"excess": excess(dq, dq32)}}
+    print("dKV at config 4:", record)
+    import json
+    import os
+    outdir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    if os.path.isdir(outdir):                                      # kept beside the run's other measurements
+        with open(os.path.join(outdir, "parity_cfg4.json"), "w") as fh:
+            json.dump(record, fh, indent=1)
     assert e32 <= FP32_DKV_EXCESS_LIMIT
+    assert e32 <= 1.6 * eref                                       # the bf16 rows add at most 60 % to the reference's excess
+    assert f32 <= 1e-3                                             # and fewer than one element in a thousand lies outside
     # and a sample of queries against the CPU oracle proper: forward, dQ by autograd
     sel = torch.tensor([0, 1, 63, 64, 2047, 2048, 5000, 8191])
     seld = sel.to(gpu)

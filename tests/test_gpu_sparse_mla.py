@@ -29,14 +29,26 @@ def test_forward_against_oracle(gpu, S, H, K, q_start, skv, seed):
 
 
 @pytest.mark.parametrize("K", [4096, 8192])
-def test_forward_with_a_top_k_beyond_2048(gpu, K):
-    """Wider slot lists run with a three-stage tile ring; the backward is limited to 2048 slots."""
+def test_top_k_beyond_2048(gpu, K):
+    """Wider slot lists: the forward runs them with a three-stage tile ring; the backward and the recomputed attention
+    distribution take 2048 / 4096 slots per call and the host walks the list in parts (the gradients are sums over the
+    slots once lse and out of the whole list are given)."""
+    from loongforge_amd import ops
+
     skv = K + 1500
     inp = O.make_mla_inputs(48, 64, K, seed=11, skv=skv, q_start=skv - 48)
     out, lse, _ = _run_fwd(inp, gpu, skv - 48)
     ro, rl, _ = O.sparse_mla_fwd(inp.q, inp.kv, inp.idx, skv - 48, inp.sm_scale, 512)
     assert_close(out, ro, "out")
     assert (lse.cpu() - rl).abs().max().item() < 1e-4
+    q, kv, ids, do = inp.q.to(gpu), inp.kv.to(gpu), inp.idx.to(gpu), inp.dout.to(gpu)
+    dq, dkv = ops.sparse_mla_bwd(q, kv, out, do, ids, lse, skv - 48, inp.sm_scale)
+    rdq, rdkv = O.sparse_mla_bwd(inp.q, inp.kv, inp.idx, inp.dout, skv - 48, inp.sm_scale, 512)
+    assert_close(dq, rdq, "dq")
+    assert_close(dkv, rdkv, "dkv")             # 48 queries: few rows per key, the bf16 rows stay inside the bound
+    dist = ops.attn_dist_qk(q, kv, ids, lse, skv - 48, inp.sm_scale, 64)
+    ref = O.attn_dist_from_lse(inp.q, inp.kv, inp.idx, rl, skv - 48, inp.sm_scale, 64)
+    assert (dist.cpu() - ref).abs().max().item() <= 2e-5
 
 
 def test_forward_p_out_and_attn_dist(gpu):
@@ -265,6 +277,19 @@ def test_backward_chunked_workspace_through_the_c_abi(gpu):
     torch.cuda.synchronize()
     assert torch.equal(dq1, dq2)
     assert (dkv1.float() - dkv2.float()).abs().max().item() <= 2 * 2.0 ** -8 * dkv1.float().abs().max().item()
+    # the smallest accepted workspace, and a repeated id in the last chunk: every chunk's dQ is NaN, not only the last's
+    least = lib.dsa_sparse_mla_bwd_workspace_bytes_min(300, 128, 300, 128)
+    assert 0 < least <= small
+    idx_dup = inp.idx.clone()
+    idx_dup[299, 5] = idx_dup[299, 9]
+    idx_dup = idx_dup.to(gpu)
+    wl = torch.empty(least, dtype=torch.uint8, device=gpu)
+    rc = lib.dsa_sparse_mla_bwd(q.data_ptr(), kv.data_ptr(), out.data_ptr(), do.data_ptr(), idx_dup.data_ptr(),
+                                lse.data_ptr(), 300, 128, 300, 128, 0, inp.sm_scale, 512, dq2.data_ptr(),
+                                dkv2.data_ptr(), wl.data_ptr(), least, None)
+    assert rc == 0, lib.dsa_last_error()
+    torch.cuda.synchronize()
+    assert torch.isnan(dq2.float()).all() and torch.isnan(dkv2.float()).all()
     tiny = torch.empty(1024, dtype=torch.uint8, device=gpu)
     rc = lib.dsa_sparse_mla_bwd(q.data_ptr(), kv.data_ptr(), out.data_ptr(), do.data_ptr(), idx.data_ptr(),
                                 lse.data_ptr(), 300, 128, 300, 128, 0, inp.sm_scale, 512, dq2.data_ptr(),

@@ -26,11 +26,15 @@ def _both(lib, gpu, S, Hi, K, seed, cu=None):
     rc = lib.dsa_indexer_topk_fwd(*args, sc_a.data_ptr(), id_a.data_ptr(), wsp.data_ptr(), nbytes, None)
     assert rc == 0, lib.dsa_last_error()
     torch.cuda.synchronize()
+    # free device memory as the driver sees it (a hipMalloc by the library would show here; torch's own
+    # counters only know torch's allocations), and torch's counter for torch's side
+    free_before, _ = torch.cuda.mem_get_info()
     before = torch.cuda.memory_allocated()
     rc = lib.dsa_indexer_topk_fwd_static(*args, sc_b.data_ptr(), id_b.data_ptr(), None)
     assert rc == 0, lib.dsa_last_error()
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after >= free_before and torch.cuda.memory_allocated() == before
     return sc_a, id_a, sc_b, id_b
 
 
