@@ -152,6 +152,7 @@ __device__ __forceinline__ void bitonic_regs(float* outv, int* outi, unsigned lo
 // the row is unsuitable (no spread, or a crowded bin): the caller then takes the general path.
 constexpr int LIN_SPARE = 960;               // extra buffer entries for the threshold bin's surplus
 constexpr int REG_ROW = 8192 + 4 * 256;      // longest row (plus alignment slack) the register variant holds
+constexpr int REG_ROW_BIG = 32768 + 4 * 256; // the same for the variant with twice the registers
 constexpr int LIN_MAX_BIN = 256;             // largest segment ranked by pairwise counting
 
 // Threshold bin of a filled histogram (thread t owns bins [PER t, PER t + PER)), then the segment
@@ -346,14 +347,18 @@ __device__ __forceinline__ bool linear_select_sort_regs(const float* __restrict_
   return true;
 }
 
-// LEAN (sorted rows that fit the register variant; implies !STAGED): the kernel keeps to 128
-// registers so that four workgroups share a compute unit; rows the single-sweep path turns down
-// take the general path on global memory and the plain LDS sorting network.
-template <bool STAGED, bool LEAN>
-__global__ __launch_bounds__(BLOCK, LEAN ? 4 : 1) void topk_kernel(const float* __restrict__ logits, long ld,
-                                                     const int* __restrict__ row_begin, const int* __restrict__ row_end,
-                                                     int width, const int* __restrict__ id_base, int K, int Kp2, int sorted,
-                                                     float* __restrict__ scores, int* __restrict__ ids, int nmax) {
+// LEAN (sorted rows held in registers; implies !STAGED).  1: rows of up to REG_ROW elements, the kernel keeps to
+// 128 registers so that four workgroups share a compute unit.  2: rows of up to REG_ROW_BIG elements at up to 256
+// registers (two workgroups per compute unit).  A launch looks only at the rows whose length lies in
+// (n_above, n_upto] and leaves the others to the launch of the other variant; rows the single-sweep path turns
+// down take the general path on global memory and the plain LDS sorting network.  Rows are taken in ascending
+// order (with causal windows the short ones first: 0.118 ms at 8192 x 8192 against 0.161 ms longest first and
+// 0.141 ms with short and long rows alternating).
+template <bool STAGED, int LEAN>
+__global__ __launch_bounds__(BLOCK, LEAN == 1 ? 4 : LEAN == 2 ? 2 : 1) void topk_kernel(
+    const float* __restrict__ logits, long ld, const int* __restrict__ row_begin, const int* __restrict__ row_end,
+    int width, const int* __restrict__ id_base, int K, int Kp2, int sorted, float* __restrict__ scores,
+    int* __restrict__ ids, int nmax, int n_above, int n_upto) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   int* hist = (int*)smem;                          // HBINS
   int* scratch = hist + HBINS;                     // 16
@@ -365,6 +370,7 @@ __global__ __launch_bounds__(BLOCK, LEAN ? 4 : 1) void topk_kernel(const float* 
   const int cb = max(row_begin ? row_begin[row] : 0, 0);
   const int ce = min(row_end ? row_end[row] : width, width);
   const int n = max(ce - cb, 0);
+  if (n <= n_above || n > n_upto) return;
   const int base_id = (id_base ? id_base[row] : 0) + cb;
   const float* src = logits + row * ld + cb;
   float* sv = scores + row * (long)K;
@@ -377,12 +383,20 @@ __global__ __launch_bounds__(BLOCK, LEAN ? 4 : 1) void topk_kernel(const float* 
     if (STAGED) {
       if (linear_select_sort(src, keys, n, K, base_id, hist, scratch, (unsigned long long*)outv, sv, si)) return;
       __syncthreads();
-    } else if (LEAN && n + 3 <= REG_ROW) {
+    } else if (LEAN == 1 && n + 3 <= REG_ROW) {
       bool done;
       unsigned long long* obuf = (unsigned long long*)outv;
       if (n + 3 <= 8 * BLOCK) done = linear_select_sort_regs<2>(src, n, K, base_id, hist, scratch, obuf, sv, si);
       else if (n + 3 <= 16 * BLOCK) done = linear_select_sort_regs<4>(src, n, K, base_id, hist, scratch, obuf, sv, si);
       else done = linear_select_sort_regs<REG_ROW / (4 * BLOCK)>(src, n, K, base_id, hist, scratch, obuf, sv, si);
+      if (done) return;
+      __syncthreads();
+    } else if (LEAN == 2 && n + 3 <= REG_ROW_BIG) {
+      bool done;
+      unsigned long long* obuf = (unsigned long long*)outv;
+      if (n + 3 <= 16 * 4 * BLOCK) done = linear_select_sort_regs<16>(src, n, K, base_id, hist, scratch, obuf, sv, si);
+      else if (n + 3 <= 24 * 4 * BLOCK) done = linear_select_sort_regs<24>(src, n, K, base_id, hist, scratch, obuf, sv, si);
+      else done = linear_select_sort_regs<REG_ROW_BIG / (4 * BLOCK)>(src, n, K, base_id, hist, scratch, obuf, sv, si);
       if (done) return;
       __syncthreads();
     }
@@ -452,7 +466,7 @@ __global__ __launch_bounds__(BLOCK, LEAN ? 4 : 1) void topk_kernel(const float* 
   __syncthreads();
 
   if (sorted) {   // bitonic sort, descending score, ascending id among equal scores
-    const int ept = LEAN ? 0 : Kp2 / BLOCK;
+    const int ept = LEAN != 0 ? 0 : Kp2 / BLOCK;
     if (ept == 8) { bitonic_regs<8>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
     else if (ept == 4) { bitonic_regs<4>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
     else if (ept == 2) { bitonic_regs<2>(outv, outi, (unsigned long long*)outv, Kp2, sv, si, K); return; }
@@ -490,15 +504,32 @@ int dsa_topk_launch(const float* logits, int S, int64_t ld, const int32_t* row_b
   while (Kp2 < K) Kp2 <<= 1;
   const size_t fixed = (size_t)HBINS * 4 + 64 + (size_t)Kp2 * 8 + (size_t)LIN_SPARE * 8;
   const size_t staged = fixed + (size_t)width * 4;
-  // sorted rows that fit the register variant need no staging buffer: four workgroups share a compute unit
-  const bool lean = sorted && width + 3 <= REG_ROW;
+  // sorted rows that fit a register variant need no staging buffer: rows of up to REG_ROW elements go to the
+  // 128-register kernel (four workgroups per compute unit), longer ones up to REG_ROW_BIG to its 256-register
+  // form in a second launch; each launch skips the other's rows
+  const bool lean = sorted && width + 3 <= REG_ROW_BIG;
   const bool use_staged = !lean && staged <= 160 * 1024;
   const size_t smem = use_staged ? staged : fixed;
-  auto kern = lean ? topk_kernel<false, true> : use_staged ? topk_kernel<true, false> : topk_kernel<false, false>;
-  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-    DSA_FAIL(DSA_ERR_LAUNCH, "dsa_topk: cannot reserve %zu bytes of LDS", smem);
-  kern<<<dim3(S), dim3(BLOCK), smem, st>>>(logits, (long)ld, row_begin, row_end, width, id_base, K, Kp2, sorted,
-                                           scores, ids, width);
+  const int none = 0x7fffffff;
+  if (lean) {
+    auto k1 = topk_kernel<false, 1>;
+    auto k2 = topk_kernel<false, 2>;
+    if (hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess ||
+        hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      DSA_FAIL(DSA_ERR_LAUNCH, "dsa_topk: cannot reserve %zu bytes of LDS", smem);
+    const int split = REG_ROW - 3;
+    k1<<<dim3(S), dim3(BLOCK), smem, st>>>(logits, (long)ld, row_begin, row_end, width, id_base, K, Kp2, sorted, scores, ids,
+                                           width, -1, split);
+    if (width > split)
+      k2<<<dim3(S), dim3(BLOCK), smem, st>>>(logits, (long)ld, row_begin, row_end, width, id_base, K, Kp2, sorted, scores,
+                                             ids, width, split, none);
+  } else {
+    auto kern = use_staged ? topk_kernel<true, 0> : topk_kernel<false, 0>;
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      DSA_FAIL(DSA_ERR_LAUNCH, "dsa_topk: cannot reserve %zu bytes of LDS", smem);
+    kern<<<dim3(S), dim3(BLOCK), smem, st>>>(logits, (long)ld, row_begin, row_end, width, id_base, K, Kp2, sorted, scores, ids,
+                                             width, -1, none);
+  }
   DSA_CHECK_LAUNCH("dsa_topk");
   return DSA_OK;
 }
@@ -517,10 +548,11 @@ int dsa_indexer_logits_block(const void* q8, const float* q_w, const void* k8, c
                              hipStream_t st);
 
 static int fused_block_rows(int Sk) {
-  // one block's logits stay within the 256 MiB memory-side cache, and a block still has enough
-  // workgroups (8 queries each) to cover all 256 compute units several times over
+  // one block's logits stay within the 256 MiB memory-side cache where that still leaves a block 8192 queries:
+  // 1024 workgroups of 8 queries, four rounds over the 256 compute units (blocks of 2048 queries - one workgroup per
+  // compute unit, half of what fits - took 2.6 ms for 32768 packed tokens where blocks of 8192 take 1.9 ms)
   long rows = (256l << 20) / ((long)Sk * 4);
-  rows = rows < 2048 ? 2048 : rows;
+  rows = rows < 8192 ? 8192 : rows;
   return (int)(rows / 8 * 8);
 }
 
