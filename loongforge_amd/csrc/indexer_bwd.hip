@@ -216,13 +216,20 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
       acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[tt][0], bk[0], acc, 0, 0, 0, 127, 0, 127);
       acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aq[tt][1], bk[1], acc, 0, 0, 0, 127, 0, 127);
 #pragma unroll
-      for (int e = 0; e < 16; e++) {
-        const float rr = acc[e];
-        dwp[tt][e] = fmaf(a, __builtin_bit_cast(float, max(__builtin_bit_cast(int, rr), 0)), dwp[tt][e]);   // relu on the bit pattern
-        const float ev = rr > 0.f ? a * wq[tt][e] : 0.f;
-        const __bf16 h = (__bf16)ev;
-        ehi[tt][e >> 3][e & 7] = h;
-        elo[tt][e >> 3][e & 7] = (__bf16)(ev - (float)h);
+      for (int e = 0; e < 16; e += 2) {
+        // two neighbouring heads at a time: one packed conversion for the bf16 heads of E, one for what they miss
+        float ev[2];
+#pragma unroll
+        for (int x = 0; x < 2; x++) {
+          const float rr = acc[e + x];
+          dwp[tt][e + x] = fmaf(a, __builtin_bit_cast(float, max(__builtin_bit_cast(int, rr), 0)), dwp[tt][e + x]);   // relu on the bit pattern
+          ev[x] = rr > 0.f ? a * wq[tt][e + x] : 0.f;
+        }
+        const unsigned ph = cvt_pk_bf16(ev[0], ev[1]);
+        const unsigned pl = cvt_pk_bf16(ev[0] - __builtin_bit_cast(float, ph << 16), ev[1] - __builtin_bit_cast(float, ph & 0xffff0000u));
+        const bf16x2 h2 = __builtin_bit_cast(bf16x2, ph), l2 = __builtin_bit_cast(bf16x2, pl);
+        ehi[tt][e >> 3][e & 7] = h2[0]; ehi[tt][e >> 3][(e & 7) + 1] = h2[1];
+        elo[tt][e >> 3][e & 7] = l2[0]; elo[tt][e >> 3][(e & 7) + 1] = l2[1];
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -278,17 +285,15 @@ __global__ __launch_bounds__(256, 1) void indexer_bwd_kernel(
       for (int c = 0; c < 4; c++) {
         const int slot16 = (4 * g + c) ^ swz(r);
         const i32x4 w = *(const i32x4*)(krow + slot16 * 16);
+        // e4m3 -> bf16 is exact; one instruction converts two bytes of a word
         bf16x8 o0, o1;
 #pragma unroll
-        for (int x = 0; x < 4; x++)
-#pragma unroll
-          for (int y = 0; y < 4; y++) {
-            const __bf16 v = (__bf16)(y == 0 ? __builtin_amdgcn_cvt_f32_fp8(w[x], 0)
-                                             : y == 1 ? __builtin_amdgcn_cvt_f32_fp8(w[x], 1)
-                                                      : y == 2 ? __builtin_amdgcn_cvt_f32_fp8(w[x], 2)
-                                                               : __builtin_amdgcn_cvt_f32_fp8(w[x], 3));
-            if (x < 2) o0[4 * x + y] = v; else o1[4 * (x - 2) + y] = v;
-          }
+        for (int x = 0; x < 4; x++) {
+          const bf16x2 lo2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[x], 1.0f, false);
+          const bf16x2 hi2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[x], 1.0f, true);
+          if (x < 2) { o0[4 * x] = lo2[0]; o0[4 * x + 1] = lo2[1]; o0[4 * x + 2] = hi2[0]; o0[4 * x + 3] = hi2[1]; }
+          else { o1[4 * (x - 2)] = lo2[0]; o1[4 * (x - 2) + 1] = lo2[1]; o1[4 * (x - 2) + 2] = hi2[0]; o1[4 * (x - 2) + 3] = hi2[1]; }
+        }
         *(bf16x8*)(kdst + (((8 * g + 2 * c) ^ ksw) << 4)) = o0;
         *(bf16x8*)(kdst + (((8 * g + 2 * c + 1) ^ ksw) << 4)) = o1;
       }
