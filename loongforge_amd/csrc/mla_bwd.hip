@@ -646,50 +646,67 @@ __device__ __forceinline__ uint4 row_load16(const void* p) {
 }
 constexpr int RED_GROUPS = 7;
 constexpr int RED_FLIGHT = 16;               // row pieces a thread has in flight
+constexpr int RED_KEYS = 4;                  // consecutive keys per workgroup
+// A workgroup sums RED_KEYS consecutive keys (their rows follow one another in the buffer): every thread walks its
+// share of the first key's rows, then of the next one's, without a barrier in between, so that the loads of one
+// key are in flight while the previous one is summed; one barrier, then the seven partial sums of each key are
+// combined.  (One key per workgroup left the per-key latencies - segment bounds, first loads, barrier, combine -
+// exposed once a key has few rows per launch: with the queries of 32768 tokens walked in four chunks the launch
+// took 27.1 ms against 18.9 ms for one sweep; per key the sums and their order are the same as before.)
 __device__ __forceinline__ void reduce_body(const unsigned char* __restrict__ rows, const int* __restrict__ start,
-                                            float* __restrict__ dkv_acc, int key, int accumulate, unsigned char* smem) {
-  float* part = (float*)smem;                  // [RED_GROUPS][DQK]
+                                            float* __restrict__ dkv_acc, int key0, int n_keys, int accumulate,
+                                            unsigned char* smem) {
+  float* part = (float*)smem;                  // [RED_KEYS][RED_GROUPS][DQK]
   const int tid = threadIdx.x;
   const int ch = tid % 72, grp = tid / 72;
-  const int s0 = start[key], s1 = start[key + 1];
-  float acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; e++) acc[e] = 0.f;
+  const int nk = min(RED_KEYS, n_keys - key0);
   if (grp < RED_GROUPS) {
-    int rr = s0 + grp;
-    for (; rr + (RED_FLIGHT - 1) * RED_GROUPS < s1; rr += RED_FLIGHT * RED_GROUPS) {
-      uint4 v[RED_FLIGHT];
+    int bounds[RED_KEYS + 1];
 #pragma unroll
-      for (int u = 0; u < RED_FLIGHT; u++) v[u] = row_load16(rows + (size_t)(rr + u * RED_GROUPS) * ROW_BYTES + ch * 16);
+    for (int k = 0; k <= RED_KEYS; k++) bounds[k] = start[min(key0 + k, n_keys)];
 #pragma unroll
-      for (int u = 0; u < RED_FLIGHT; u++) {
-        const unsigned w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+    for (int k = 0; k < RED_KEYS; k++) {
+      if (k >= nk) break;
+      const int s0 = bounds[k], s1 = bounds[k + 1];
+      float acc[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc[e] = 0.f;
+      int rr = s0 + grp;
+      for (; rr + (RED_FLIGHT - 1) * RED_GROUPS < s1; rr += RED_FLIGHT * RED_GROUPS) {
+        uint4 v[RED_FLIGHT];
+#pragma unroll
+        for (int u = 0; u < RED_FLIGHT; u++) v[u] = row_load16(rows + (size_t)(rr + u * RED_GROUPS) * ROW_BYTES + ch * 16);
+#pragma unroll
+        for (int u = 0; u < RED_FLIGHT; u++) {
+          const unsigned w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            acc[2 * e] += __builtin_bit_cast(float, w[e] << 16);
+            acc[2 * e + 1] += __builtin_bit_cast(float, w[e] & 0xffff0000u);
+          }
+        }
+      }
+      for (; rr < s1; rr += RED_GROUPS) {
+        const uint4 v = row_load16(rows + (size_t)rr * ROW_BYTES + ch * 16);
+        const unsigned w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           acc[2 * e] += __builtin_bit_cast(float, w[e] << 16);
           acc[2 * e + 1] += __builtin_bit_cast(float, w[e] & 0xffff0000u);
         }
       }
-    }
-    for (; rr < s1; rr += RED_GROUPS) {
-      const uint4 v = row_load16(rows + (size_t)rr * ROW_BYTES + ch * 16);
-      const unsigned w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        acc[2 * e] += __builtin_bit_cast(float, w[e] << 16);
-        acc[2 * e + 1] += __builtin_bit_cast(float, w[e] & 0xffff0000u);
-      }
+      for (int e = 0; e < 8; e++) part[(k * RED_GROUPS + grp) * DQK + ch * 8 + e] = acc[e];
     }
-#pragma unroll
-    for (int e = 0; e < 8; e++) part[grp * DQK + ch * 8 + e] = acc[e];
   }
   __syncthreads();
-  for (int d = tid; d < DQK; d += (int)blockDim.x) {
-    float s = part[d];
+  for (int o = tid; o < nk * DQK; o += (int)blockDim.x) {
+    const int k = o / DQK, d = o % DQK;
+    float sum = part[k * RED_GROUPS * DQK + d];
 #pragma unroll
-    for (int gq = 1; gq < RED_GROUPS; gq++) s += part[gq * DQK + d];
-    float* p = dkv_acc + (size_t)key * DQK + d;
-    *p = accumulate ? *p + s : s;
+    for (int gq = 1; gq < RED_GROUPS; gq++) sum += part[(k * RED_GROUPS + gq) * DQK + d];
+    float* p = dkv_acc + (size_t)(key0 + k) * DQK + d;
+    *p = accumulate ? *p + sum : sum;
   }
 }
 
@@ -698,12 +715,10 @@ __device__ __forceinline__ void reduce_body(const unsigned char* __restrict__ ro
 // ---------------------------------------------------------------------------------------------
 // Pass B is bound by LDS reads and leaves HBM nearly idle; pass D is a pure stream of HBM reads and
 // leaves everything else idle; each occupies a whole compute unit (140 KB of LDS, or all its
-// memory-level parallelism).  One launch carries the workgroups of both, alternating in dispatch
-// order, so that at any time about half of the compute units work on either:
+// memory-level parallelism).  One launch carries the workgroups of both, spread evenly over the
+// dispatch order, so that both kinds of work are in flight from the first workgroup to the last:
 //   bwd_dq_reduce_kernel   pass B of all queries | pass D of all keys      (4.5 ms against 2.6 + 2.75)
-// Workgroup b of a launch with nX and nY workgroups of the two roles: the first 2*min(nX, nY)
-// alternate (even b: X), the rest belong to the longer role.  Within a role, the longest work
-// (latest query, earliest key) comes first.
+// Within a role, the longest work (latest query, earliest key) comes first.
 // Passes A and C, carried by one launch in the same way (pass A of one block of queries beside
 // pass C of the block before it, 2 - 64 interleaved blocks), took as long side by side as one after
 // the other: neither gets faster when it has fewer compute units - a compute unit that alternates
@@ -711,10 +726,13 @@ __device__ __forceinline__ void reduce_body(const unsigned char* __restrict__ ro
 // other, which bounds pass C per compute unit at about the rate at which HBM bounds it for the
 // whole chip.  They are separate kernels.
 struct RoleSlot { bool first; int i; };
+// nX workgroups of the first role and nY of the second, spread evenly over the launch: workgroup b belongs to the
+// second role when the count floor(b * nY / (nX + nY)) steps up after it.
 __device__ __forceinline__ RoleSlot role_slot(int b, int nX, int nY) {
-  const int n2 = nX < nY ? nX : nY;
-  if (b < 2 * n2) return {(b & 1) == 0, b >> 1};
-  return {nX > nY, n2 + (b - 2 * n2)};
+  const long long tot = (long long)nX + nY;
+  const int y0 = (int)((long long)b * nY / tot), y1 = (int)((long long)(b + 1) * nY / tot);
+  if (y1 > y0) return {false, y0};
+  return {true, b - y0};
 }
 
 __global__ __launch_bounds__(PDS_THREADS, 1) void bwd_pds_kernel(
@@ -743,9 +761,9 @@ __global__ __launch_bounds__(DQ_THREADS, 1) void bwd_dq_reduce_kernel(
     const unsigned char* __restrict__ rows, const int* __restrict__ start, float* __restrict__ dkv_acc, int n_keys,
     int accumulate) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  const RoleSlot rs = role_slot((int)blockIdx.x, cnt, n_keys);
+  const RoleSlot rs = role_slot((int)blockIdx.x, cnt, (n_keys + RED_KEYS - 1) / RED_KEYS);
   if (rs.first) dq_body<3>(kv, ids, pds, dq, q0, cnt - 1 - rs.i, H, Skv, K, q_start, dup_flag, smem);
-  else reduce_body(rows, start, dkv_acc, rs.i, accumulate, smem);
+  else reduce_body(rows, start, dkv_acc, rs.i * RED_KEYS, n_keys, accumulate, smem);
 }
 
 // fp32 accumulator -> bf16 dKV; NaN everywhere when a query row held a repeated id
@@ -896,7 +914,7 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dKV rows)");
     DSA_MARK(3);
     // Pass B of every query beside pass D of every key.
-    bwd_dq_reduce_kernel<<<dim3(cnt + Skv), dim3(DQ_THREADS), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv,
+    bwd_dq_reduce_kernel<<<dim3(cnt + (Skv + RED_KEYS - 1) / RED_KEYS), dim3(DQ_THREADS), smemB, st>>>((const __bf16*)kv, sids, pds, (__bf16*)dq, q0, cnt, H, Skv,
                                                                    K, q_start, dup_flag, rows, start, acc, Skv, first ? 0 : 1);
     DSA_CHECK_LAUNCH("dsa_sparse_mla_bwd(dQ | dKV reduce)");
     DSA_MARK(4);
