@@ -331,9 +331,11 @@ class DSAIndexerFused(MegatronModule):
         mscale = 1.0
         cos = sin = None
         if getattr(self.config, "apply_rope_fusion", False):
-            if chunkpipe:
-                raise NotImplementedError("chunkpipe with apply_rope_fusion: the cached cos / sin tables carry no offset")
-            cos, sin = self.rotary_pos_emb.get_cached_cos_sin(rotary_seq_len, dtype=x.dtype, packed_seq=packed_seq)
+            # the fused kernel indexes its tables by the token's place in this call: a chunk reads the tables of
+            # the sequence so far from its own first position on
+            cos, sin = self.rotary_pos_emb.get_cached_cos_sin(pos_emb_offset + rotary_seq_len, dtype=x.dtype,
+                                                              packed_seq=packed_seq)
+            cos, sin = cos[pos_emb_offset:].contiguous(), sin[pos_emb_offset:].contiguous()
         if packed_seq_params is not None:
             cu_seqlens_q = packed_seq_params.cu_seqlens_q_padded
             if cu_seqlens_q is None:

@@ -157,3 +157,59 @@ def test_absorbed_mla_module_packed_and_fused_equals_unfused(gpu):
     assert (y1.float() - y2.float()).abs().max().item() <= 2e-2 * y2.float().abs().max().item()
     ref = M.mla_dense(x[100:, 0].double().cpu(), {k: v.double() for k, v in _weights(fused).items()}, H)
     assert (y1[100:, 0].double().cpu() - ref).abs().max().item() <= 2e-2 * ref.abs().max().item()
+
+
+@pytest.mark.parametrize("fusion", [False, True])
+def test_chunkpipe_through_the_mla_module_matches_the_whole_sequence(gpu, fusion):
+    """Chunkpipe at the level of the attention module (multi_latent_attention.py:468-555, :921-922, :1058-1064,
+    :1274-1298 of the reference): the sequence arrives in chunks; every chunk caches its normalised latent and its
+    rotated key position channels, attends to [cached | own] keys at their positions in the whole sequence, and the
+    gradient it sends to cached keys reaches the producing chunk's backward (run last chunk first).  Outputs and
+    weight gradients must agree with the same module run on the whole sequence; top-k covers the sequence, so the
+    selection cannot differ."""
+    import copy
+
+    C, cs, H, hid, qlr = 3, 64, 16, 128, 96
+    S = C * cs
+    whole = _module(gpu, fusion, S, H, hid, qlr, topk=256).train()
+    chunked = copy.deepcopy(whole)
+    cfg = copy.copy(whole.config)
+    cfg.__dict__.update(enable_chunkpipe=True, chunk_num_per_seq=C, chunksize=cs, micro_batch_size=1, chunkpipe_forward=True,
+                        chunkpipe_forward_microbatch=0, chunkpipe_backward_microbatch=0, keep_activations_chunks=C,
+                        virtual_pipeline_model_parallel_size=None)
+    chunked.config = chunked.core_attention.config = chunked.core_attention.indexer.config = cfg
+    chunked.init_chunk_key_value_cache_mla()
+    chunked.core_attention.indexer.setup_chunkpipe_indexer_cache_config()
+    chunked.core_attention.indexer.init_chunk_indexer_key_cache()
+    chunked = chunked.to(gpu)
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(S, 1, hid, generator=g).to(torch.bfloat16).to(gpu)
+    gy = torch.randn(S, 1, hid, generator=g).to(torch.bfloat16).to(gpu)
+    y_w, _ = whole(x, None)
+    y_w.backward(gy)
+    outs = []
+    for c in range(C):
+        cfg.chunkpipe_forward_microbatch = c
+        assert chunked.is_enable_grad_chunkpipe()
+        y_c, _ = chunked(x[c * cs:(c + 1) * cs], None)
+        outs.append(y_c)
+        ref = y_w[c * cs:(c + 1) * cs].float()
+        assert (y_c.float() - ref).abs().max().item() <= 2e-2 * ref.abs().max().item()
+    assert len(chunked.micro_batch_to_cache_chunk_map) == C - 1           # the last chunk is not cached
+    for c in reversed(range(C)):
+        outs[c].backward(gy[c * cs:(c + 1) * cs])
+    assert not chunked.kv_compressed_cache_grad and not chunked.key_pos_emb_cache_grad
+    for (n, pw), pc in zip(whole.named_parameters(), chunked.parameters()):
+        if pw.grad is None:
+            assert pc.grad is None or "indexer" in n, n
+            continue
+        scale = pw.grad.abs().max().item()
+        err = (pc.grad - pw.grad).abs().max().item()
+        assert err <= 4e-2 * scale, "%s: %.3e against %.3e" % (n, err, scale)
+    # the schedule's calls and their guards
+    chunked.delete_chunk_key_value_cache(0)
+    assert len(chunked.micro_batch_to_cache_chunk_map) == C - 2
+    chunked.clear_chunk_key_value_cache()
+    assert not chunked.micro_batch_to_cache_chunk_map
+    with pytest.raises(RuntimeError):
+        whole.concat_cached_chunk_key_value_dsa(x)
