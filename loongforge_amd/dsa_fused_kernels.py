@@ -92,13 +92,21 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
             if attn_sink.numel() != h_q:
                 attn_sink = attn_sink.flatten().repeat_interleave(h_q // attn_sink.numel())
             attn_sink = attn_sink.contiguous().view(h_q).float()
-        # the head-averaged distribution comes from materialised logits when they are small enough to be a
-        # passing allocation (forward + 0.9 ms, reduction 0.8 ms at 8k tokens x 128 heads x 2048 slots: 4.3 GB),
-        # and is recomputed from q, kv and lse otherwise (2.7 ms, no [sq, n, topk] tensor: 17 GB at 32k tokens)
-        dist_from_logits = (bool(dist_heads) and
-                            sq * q.size(1) * ids.shape[-1] * 2 <= float(os.environ.get("DSA_P_OUT_BUDGET_GIB", "6")) * 2 ** 30)
-        out, lse, p_out = ops.sparse_mla_fwd(q, kv2, ids, chunk_offset, sm_scale, d_v, return_p_out or dist_from_logits,
-                                             attn_sink=attn_sink, p_out_skip=window_size)
+        # the head-averaged distribution comes from the forward's raw logits, which are a passing buffer of at most
+        # DSA_P_OUT_BUDGET_GIB (default 6) GiB: all queries at once when they fit (forward + 0.9 ms, reduction 0.8 ms at
+        # 8k tokens x 128 heads x 2048 slots: 4.3 GB), else a block of queries at a time (17 GB of logits at 32k tokens
+        # never exist; recomputing the distribution from q, kv and lse instead costs 2.6 ms per 8k tokens)
+        budget = float(os.environ.get("DSA_P_OUT_BUDGET_GIB", "6")) * 2 ** 30
+        per_query = q.size(1) * ids.shape[-1] * 2
+        dist = None
+        if dist_heads and not return_p_out and sq * per_query > budget and budget >= 64 * per_query:
+            out, lse, dist = ops.sparse_mla_fwd_dist(q, kv2, ids, chunk_offset, sm_scale, d_v, int(dist_heads),
+                                                     int(budget // per_query) // 64 * 64, attn_sink)
+            p_out = None
+        else:
+            dist_from_logits = bool(dist_heads) and sq * per_query <= budget
+            out, lse, p_out = ops.sparse_mla_fwd(q, kv2, ids, chunk_offset, sm_scale, d_v, return_p_out or dist_from_logits,
+                                                 attn_sink=attn_sink, p_out_skip=window_size)
         ctx.save_for_backward(q, kv, ids, out, lse)
         ctx.sm_scale = sm_scale
         ctx.chunk_offset = chunk_offset
@@ -108,7 +116,9 @@ class DSADotProductAttentionFunction(torch.autograd.Function):
             ctx.mark_non_differentiable(p_out)
             return out, p_out
         if dist_heads:
-            if dist_from_logits:
+            if dist is not None:
+                pass
+            elif dist_from_logits:
                 dist = ops.attn_dist(p_out[:, :int(dist_heads)], sm_scale)
                 del p_out
             else:

@@ -446,6 +446,51 @@ def sparse_mla_fwd(q, kv, ids, q_start: int = 0, sm_scale: Optional[float] = Non
     return out, lse, (p_out if return_p_out else None)
 
 
+@torch.library.custom_op("dsa::sparse_mla_fwd_dist", mutates_args=())
+def _mla_fwd_dist_op(q: torch.Tensor, kv: torch.Tensor, ids: torch.Tensor, q_start: int, sm_scale: float, d_v: int,
+                     dist_heads: int, block: int, attn_sink: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _check_mla(q, kv, ids)
+    q, kv, ids = _c(q), _c(kv), _c(ids.int())
+    S, H, _ = q.shape
+    K = ids.shape[1]
+    if attn_sink is not None:
+        _need_gpu(attn_sink)
+        attn_sink = _c(attn_sink.float().reshape(H))
+    out = torch.empty(S, H, d_v, dtype=torch.bfloat16, device=q.device)
+    lse = torch.empty(S, H, dtype=torch.float32, device=q.device)
+    dist = torch.empty(S, K, dtype=torch.float32, device=q.device)
+    block = max(1, min(int(block), S))
+    p_out = torch.empty(block, H, K, dtype=torch.bfloat16, device=q.device)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        st = _stream(q)
+        for s0 in range(0, S, block):
+            n = min(block, S - s0)
+            _lib.check(lib.dsa_sparse_mla_fwd_ex(q[s0:].data_ptr(), kv.data_ptr(), ids[s0:].data_ptr(), n, H, kv.shape[0], K,
+                                                 int(q_start) + s0, float(sm_scale), int(d_v), out[s0:].data_ptr(),
+                                                 lse[s0:].data_ptr(), p_out.data_ptr(), 0,
+                                                 attn_sink.data_ptr() if attn_sink is not None else None, 0, st),
+                       "dsa_sparse_mla_fwd")
+            _lib.check(lib.dsa_attn_dist(p_out.data_ptr(), 0, n, int(dist_heads), K, H * K, K, float(sm_scale),
+                                         dist[s0:].data_ptr(), st), "dsa_attn_dist")
+    return out, lse, dist
+
+
+@_mla_fwd_dist_op.register_fake
+def _(q, kv, ids, q_start, sm_scale, d_v, dist_heads, block, attn_sink=None):
+    S, H, _ = q.shape
+    return q.new_empty(S, H, d_v), q.new_empty(S, H, dtype=torch.float32), q.new_empty(S, ids.shape[1], dtype=torch.float32)
+
+
+def sparse_mla_fwd_dist(q, kv, ids, q_start: int, sm_scale: float, d_v: int, dist_heads: int, block: int,
+                        attn_sink: Optional[torch.Tensor] = None):
+    """(out, lse, dist): the forward together with the head-averaged attention distribution over the first
+    ``dist_heads`` heads (``attn_dist`` of the forward's raw logits), ``block`` queries at a time, so that the logits
+    ``[block, H, K]`` are a passing buffer whatever the number of queries (a block's forward writes them, the
+    reduction reads them back while they are still in the caches)."""
+    return _mla_fwd_dist_op(q, kv, ids, int(q_start), float(sm_scale), int(d_v), int(dist_heads), int(block), attn_sink)
+
+
 _BWD_WS = {}      # device index -> workspace kept between calls
 BWD_MAX_SLOTS = 2048      # slots per query the backward kernels take in one call
 ATTN_DIST_QK_MAX_SLOTS = 4096

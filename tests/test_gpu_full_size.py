@@ -252,10 +252,12 @@ def test_config1_tiny_dsa_forward_at_its_stated_size(gpu):
     assert_close(out[0, :, :H], ref["out"], "out")
     target = ops.attn_dist(p_out[:, :H], sm)
     assert (target.cpu() - ref["target"]).abs().max().item() <= 2e-3           # the logits pass through bf16
-    # return_attn_dist: from the logits while those stay under the byte budget (bf16 logits), recomputed from
-    # q, kv and lse beyond it (fp32 throughout)
+    # return_attn_dist: from the logits while those stay under the byte budget (bf16 logits); beyond it from the logits
+    # of a block of queries at a time (here four blocks of 256: bit for bit the same), and recomputed from q, kv and lse
+    # (fp32 throughout) when the budget does not even hold 64 queries
     import os
-    for budget, tol in (("6", 2e-3), ("0", 5e-5)):
+    seen = {}
+    for budget, tol in (("6", 2e-3), ("0.015625", 2e-3), ("0", 5e-5)):
         os.environ["DSA_P_OUT_BUDGET_GIB"] = budget
         try:
             out2, target2 = attn(q_pad.unsqueeze(1), kv.to(gpu).unsqueeze(1), ref_ids.unsqueeze(0), 0, AttnMaskType.causal,
@@ -264,5 +266,7 @@ def test_config1_tiny_dsa_forward_at_its_stated_size(gpu):
             del os.environ["DSA_P_OUT_BUDGET_GIB"]
         assert torch.equal(out2, out)
         assert (target2.cpu() - ref["target"]).abs().max().item() <= tol
+        seen[budget] = target2
+    assert torch.equal(seen["6"], seen["0.015625"])
     loss = O.indexer_kl_loss(ref["scores"], target2.cpu(), 1.0, S)
     assert abs(loss.item() - ref["loss"].item()) <= 1e-3 * abs(ref["loss"].item()) + 1e-6
