@@ -76,7 +76,8 @@ int dsa_quant_rowwise_e4m3_weights(const void* x, int64_t rows, int cols, void* 
  * sin indexing of dsa_rope_rows with equal source and destination pairing (0 adjacent pairs, 1 split pairs
  * (i, i + 32), -1 none): fused_apply_mla_rope(..., pe_first=True), dsa_fused.py:435-451.
  *   x [rows, 128] bf16, rows = tokens * rows_per_token; position of a row's token: positions[token], or
- *   token / batch when positions is NULL; cos, sin [max position + 1, 64] bf16 or f32 (cos_sin_f32);
+ *   token / batch when positions is NULL; cos, sin [max position + 1, 64] bf16 or f32 (cos_sin_f32): the tables must
+ *   reach the largest position given - the entry point does not know their length and checks nothing there;
  *   ln_weight, ln_bias [128] f32 or both NULL (no LayerNorm); rotate != 0 applies the Hadamard rotation.
  *   Outputs as dsa_rotate_quant_e4m3 (x8 / scale_inv and / or y) and dsa_quant_rowwise_e4m3_weights
  *   (weights, weight_scaled [rows] f32, or both NULL).
