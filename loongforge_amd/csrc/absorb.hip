@@ -93,7 +93,7 @@ int launch(const void* a, int64_t a_tok, int64_t a_head, const void* w, void* c,
   auto kern = absorb_kernel<K, N>;
   static bool configured = false;            // per template instance
   if (!configured) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2;
+    if (dsa_reserve_lds((const void*)kern, smem) != hipSuccess) return -2;
     configured = true;
   }
   kern<<<dim3((unsigned)(H * splits)), dim3(256), smem, st>>>((const __bf16*)a, (long)a_tok, (long)a_head, (const __bf16*)w,

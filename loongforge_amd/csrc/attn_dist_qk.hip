@@ -128,7 +128,7 @@ extern "C" int dsa_attn_dist_qk(const void* q, const void* kv, const int32_t* id
   const int stages = (size_t)3 * TILE_BYTES + tail <= 160 * 1024 ? 3 : 2;
   const size_t smem = (size_t)stages * TILE_BYTES + tail;
   auto kern = stages == 3 ? attn_dist_qk_kernel<3> : attn_dist_qk_kernel<2>;
-  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+  if (dsa_reserve_lds((const void*)kern, smem) != hipSuccess)
     DSA_FAIL(DSA_ERR_LAUNCH, "dsa_attn_dist_qk: cannot reserve %zu bytes of LDS", smem);
   kern<<<dim3(S), dim3(256), smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, lse, target, H, heads_in_mean, Skv, K,
                                          q_start, sm_scale);

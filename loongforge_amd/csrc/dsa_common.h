@@ -26,6 +26,10 @@ void dsa_set_error(const char* fmt, ...);
 #define DSA_CHECK_LAUNCH(name) do { hipError_t e_ = hipGetLastError(); \
     if (e_ != hipSuccess) DSA_FAIL(DSA_ERR_LAUNCH, "%s: launch failed: %s", name, hipGetErrorString(e_)); } while (0)
 
+// hipFuncSetAttribute(fn, MaxDynamicSharedMemorySize, bytes), once per kernel and device while `bytes` does not
+// grow: the call costs several microseconds of host time, which a short kernel sequence cannot hide.
+hipError_t dsa_reserve_lds(const void* fn, size_t bytes);
+
 // ---- small device helpers ----------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned short h) {
   return __builtin_bit_cast(float, ((unsigned)h) << 16);

@@ -473,7 +473,7 @@ extern "C" int dsa_indexer_bwd(const float* g, const void* q8, const void* k8, c
   const size_t red_bytes = (size_t)Hi * RED_STRIDE * 4;
   if (red_bytes > (size_t)2 * TILE_BYTES + 4 * 32 * 256) smem += red_bytes;
   auto kern = Hi == 32 ? indexer_bwd_kernel<1> : indexer_bwd_kernel<2>;
-  if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+  if (dsa_reserve_lds((const void*)kern, smem) != hipSuccess)
     DSA_FAIL(DSA_ERR_LAUNCH, "dsa_indexer_bwd: cannot reserve LDS");
   bool first = true;
   order::clear_flag(dup_flag, st);

@@ -873,9 +873,9 @@ static int bwd_impl(const void* q, const void* kv, const void* out, const void* 
   const size_t smemA = (size_t)4 * TILE_BYTES + ids_lds_bytes(K) + 16 + 1024;
   const size_t smemB = (size_t)3 * (TILE_BYTES + PDS_KIND_BYTES) + ids_lds_bytes(K);
   const size_t smemC = (size_t)DKV_COEF_STAGES * PDS_TILE_BYTES + ids_lds_bytes(K) + 16 + (size_t)(K + BI) * 4;
-  if (hipFuncSetAttribute((const void*)bwd_pds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemA) != hipSuccess ||
-      hipFuncSetAttribute((const void*)bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemC) != hipSuccess ||
-      hipFuncSetAttribute((const void*)bwd_dq_reduce_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smemB) != hipSuccess)
+  if (dsa_reserve_lds((const void*)bwd_pds_kernel, smemA) != hipSuccess ||
+      dsa_reserve_lds((const void*)bwd_dkv_kernel, smemC) != hipSuccess ||
+      dsa_reserve_lds((const void*)bwd_dq_reduce_kernel, smemB) != hipSuccess)
     DSA_FAIL(DSA_ERR_LAUNCH, "dsa_sparse_mla_bwd: cannot reserve LDS");
 
   // optional timing (profiling entry point only): events between the launch groups

@@ -336,8 +336,8 @@ int launch_fwd(const void* q, const void* kv, const int32_t* ids, int S, int H, 
 #define DSA_FWD_LAUNCH(P) do { \
     auto kern = mla_fwd_kernel<STAGES, P, false>; \
     auto kern2 = mla_fwd_kernel<STAGES, P, true>; \
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2; \
-    if (hipFuncSetAttribute((const void*)kern2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) return -2; \
+    if (dsa_reserve_lds((const void*)kern, smem) != hipSuccess) return -2; \
+    if (dsa_reserve_lds((const void*)kern2, smem) != hipSuccess) return -2; \
     kern<<<grid, block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip); \
     kern2<<<dim3((S + 31) / 32), block, smem, st>>>((const __bf16*)q, (const __bf16*)kv, ids, (__bf16*)out, lse, p_out, S, H, Skv, K, q_start, sm_scale, sink, p_skip); \
   } while (0)

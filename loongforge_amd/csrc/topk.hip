@@ -514,8 +514,8 @@ int dsa_topk_launch(const float* logits, int S, int64_t ld, const int32_t* row_b
   if (lean) {
     auto k1 = topk_kernel<false, 1>;
     auto k2 = topk_kernel<false, 2>;
-    if (hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess ||
-        hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+    if (dsa_reserve_lds((const void*)k1, smem) != hipSuccess ||
+        dsa_reserve_lds((const void*)k2, smem) != hipSuccess)
       DSA_FAIL(DSA_ERR_LAUNCH, "dsa_topk: cannot reserve %zu bytes of LDS", smem);
     const int split = REG_ROW - 3;
     k1<<<dim3(S), dim3(BLOCK), smem, st>>>(logits, (long)ld, row_begin, row_end, width, id_base, K, Kp2, sorted, scores, ids,
@@ -525,7 +525,7 @@ int dsa_topk_launch(const float* logits, int S, int64_t ld, const int32_t* row_b
                                              ids, width, split, none);
   } else {
     auto kern = use_staged ? topk_kernel<true, 0> : topk_kernel<false, 0>;
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+    if (dsa_reserve_lds((const void*)kern, smem) != hipSuccess)
       DSA_FAIL(DSA_ERR_LAUNCH, "dsa_topk: cannot reserve %zu bytes of LDS", smem);
     kern<<<dim3(S), dim3(BLOCK), smem, st>>>(logits, (long)ld, row_begin, row_end, width, id_base, K, Kp2, sorted, scores, ids,
                                              width, -1, none);
