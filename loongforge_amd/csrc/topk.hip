@@ -280,15 +280,15 @@ __device__ __forceinline__ bool linear_select_sort(const float* __restrict__ src
 // The same for rows of at most 4 NV BLOCK elements, with the row held in registers instead of
 // LDS: thread t owns the 16-byte chunks t, t + BLOCK, ... of the row counted from the 16-byte
 // boundary at or below its first element, so the whole row is fetched by NV vector loads issued
-// together and the workgroup needs only the histogram and the output buffer in LDS.
+// together and the workgroup needs only the histogram and the output buffer in LDS.  The row is
+// positions [off, m) of that layout; chunk i (positions [4 BLOCK i, 4 BLOCK (i + 1))) is touched only
+// while it holds any of them.
 template <int NV>
-__device__ __forceinline__ bool linear_select_sort_regs(const float* __restrict__ src, int n, int K, int base_id,
-                                                        int* hist, int* scratch, unsigned long long* obuf, float* sv, int* si) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int off = (int)(((uintptr_t)src >> 2) & 3);        // elements between that boundary and src
+__device__ __forceinline__ void load_row_regs(const float* __restrict__ src, int n, float (&v)[NV][4], int& off, int& m) {
+  const int tid = threadIdx.x;
+  off = (int)(((uintptr_t)src >> 2) & 3);                  // elements between that boundary and src
   const float* base = src - off;
-  const int m = n + off;                                    // the row is [off, m) of base
-  float v[NV][4];
+  m = n + off;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const int p = 4 * (tid + BLOCK * i);
@@ -300,6 +300,110 @@ __device__ __forceinline__ bool linear_select_sort_regs(const float* __restrict_
       for (int j = 0; j < 4; j++) v[i][j] = (p + j >= off && p + j < m) ? base[p + j] : -INFINITY;
     }
   }
+}
+
+// min / max of three without the canonicalising v_max that fminf / fmaxf put in front of every operand
+__device__ __forceinline__ float min3_raw(float a, float b, float c) {
+  float r;
+  asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// The selection itself for rows whose values are all finite - the common case.  No per-element
+// finiteness tests (an infinity shows in the row's minimum or maximum, a NaN in one unordered compare
+// per two elements), min / max three at a time, bins without a clamp ((mx - x) scale < HBINS for every
+// x in [mn, mx]), and chunks wholly inside the row need no position tests.  Returns 1 when the row is
+// done, 0 when it is unsuitable (no spread, a crowded bin), -1 when it holds a non-finite value (the
+// caller then runs the tolerant form below on the same registers).
+template <int NV>
+__device__ __forceinline__ int select_regs_finite(const float (&v)[NV][4], int off, int m, int K, int base_id, int* hist,
+                                                  int* scratch, unsigned long long* obuf, float* sv, int* si) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int CH = 4 * BLOCK;
+  const int nch = (m + CH - 1) / CH;                        // chunks that hold any of the row
+  auto chunk_full = [&](int i) { return (i > 0 || off == 0) && CH * (i + 1) <= m; };   // the same for all threads
+  for (int b = tid; b < HBINS; b += BLOCK) hist[b] = 0;
+  float mn = INFINITY, mx = -INFINITY;
+  bool nan = false;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    if (i >= nch) continue;
+    if (chunk_full(i)) {
+      mn = min3_raw(mn, v[i][0], v[i][1]); mn = min3_raw(mn, v[i][2], v[i][3]);
+      mx = max3_raw(mx, v[i][0], v[i][1]); mx = max3_raw(mx, v[i][2], v[i][3]);
+      nan |= __builtin_isunordered(v[i][0], v[i][1]) | __builtin_isunordered(v[i][2], v[i][3]);
+    } else {
+      const int p = 4 * (tid + BLOCK * i);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (p + j >= off && p + j < m) {
+          mn = min3_raw(mn, v[i][j], v[i][j]); mx = max3_raw(mx, v[i][j], v[i][j]);
+          nan |= v[i][j] != v[i][j];
+        }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  const bool wave_nan = __ballot(nan) != 0ull;
+  if (lane == 0) { ((float*)scratch)[wave] = mn; ((float*)scratch)[4 + wave] = mx; scratch[8 + wave] = wave_nan; }
+  __syncthreads();
+  mn = fminf(fminf(((float*)scratch)[0], ((float*)scratch)[1]), fminf(((float*)scratch)[2], ((float*)scratch)[3]));
+  mx = fmaxf(fmaxf(((float*)scratch)[4], ((float*)scratch)[5]), fmaxf(((float*)scratch)[6], ((float*)scratch)[7]));
+  const bool any_nan = (scratch[8] | scratch[9] | scratch[10] | scratch[11]) != 0;
+  __syncthreads();
+  if (any_nan || !(mn > -INFINITY) || !(mx < INFINITY)) return -1;
+  const float span = mx - mn;
+  if (!(span > 0.f) || !(span < INFINITY)) return 0;
+  const int keff = min(K, m - off);
+  const float scale = ((float)HBINS - 0.5f) / span;
+  auto bin_of = [&](float x) { return (int)((mx - x) * scale); };
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    if (i >= nch) continue;
+    if (chunk_full(i)) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) atomicAdd(&hist[bin_of(v[i][j])], 1);
+    } else {
+      const int p = 4 * (tid + BLOCK * i);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (p + j >= off && p + j < m) atomicAdd(&hist[bin_of(v[i][j])], 1);
+    }
+  }
+  __syncthreads();
+  int tbin, above, c;
+  if (!lin_threshold(hist, scratch, keff, tbin, above, c)) return 0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    if (i >= nch) continue;
+    const int p = 4 * (tid + BLOCK * i);
+    const bool full = chunk_full(i);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (full || (p + j >= off && p + j < m)) {
+        const int b = bin_of(v[i][j]);
+        if (b <= tbin) obuf[atomicAdd(&hist[b], 1)] = sort_key(v[i][j], p + j - off);
+      }
+  }
+  __syncthreads();
+  lin_rank(obuf, hist, above + c, keff, K, base_id, bin_of, sv, si);
+  return 1;
+}
+
+// The tolerant form: values that are not finite (-inf marks a column that cannot be selected) are skipped
+// one by one.
+template <int NV>
+__device__ __forceinline__ bool select_regs_tolerant(const float (&v)[NV][4], int off, int K, int base_id, int* hist,
+                                                     int* scratch, unsigned long long* obuf, float* sv, int* si) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int b = tid; b < HBINS; b += BLOCK) hist[b] = 0;
   float mn = INFINITY, mx = -INFINITY;
   int nfin = 0;
@@ -345,6 +449,18 @@ __device__ __forceinline__ bool linear_select_sort_regs(const float* __restrict_
   __syncthreads();
   lin_rank(obuf, hist, above + c, keff, K, base_id, bin_of, sv, si);
   return true;
+}
+
+template <int NV>
+__device__ __forceinline__ bool linear_select_sort_regs(const float* __restrict__ src, int n, int K, int base_id,
+                                                        int* hist, int* scratch, unsigned long long* obuf, float* sv, int* si) {
+  float v[NV][4];
+  int off, m;
+  load_row_regs<NV>(src, n, v, off, m);
+  const int r = select_regs_finite<NV>(v, off, m, K, base_id, hist, scratch, obuf, sv, si);
+  if (r >= 0) return r == 1;
+  __syncthreads();
+  return select_regs_tolerant<NV>(v, off, K, base_id, hist, scratch, obuf, sv, si);
 }
 
 // LEAN (sorted rows held in registers; implies !STAGED).  1: rows of up to REG_ROW elements, the kernel keeps to
