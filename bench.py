@@ -167,7 +167,7 @@ def config_row(n):
             out, lse, target = ops.sparse_mla_fwd_dist(q, kv, ids, 0, sm, DV, H, 12288)
             ev[2].record()
             scg = sc.detach().requires_grad_(True)
-            O.indexer_kl_loss(scg, target, 1.0, T).backward()
+            (ops.indexer_kl_loss(scg, target) * (1.0 / T)).backward()
             gs = torch.where(ids >= 0, scg.grad, torch.zeros_like(sc)).contiguous()
             ev[3].record()
             ops.indexer_bwd(gs, q8, k8, ksc, ws, ids)

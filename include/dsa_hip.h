@@ -217,6 +217,18 @@ int dsa_sparse_mla_bwd(const void* q, const void* kv, const void* out, const voi
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * KL loss of the indexer's scores against the attention distribution, and its gradient, per query row:
+ *   pred = softmax_t(scores[i,:])    u = target[i,:] + eps
+ *   row_loss[i] = sum_t u_t (log u_t - log(pred_t + eps))      grad[i,t] = d row_loss[i] / d scores[i,t]
+ * sum_i row_loss[i] is F.kl_div((pred + eps).log(), target + eps, reduction="sum") of
+ * dsa_fused.py:931-944 (eps = 1e-10 there); padded slots (score -inf, target 0) add nothing and get
+ * gradient 0.  `ld_s` / `ld_t` are the row strides of scores / target in elements.
+ *   scores [S, K] f32   target [S, K] f32   row_loss [S] f32   grad [S, K] f32
+ */
+int dsa_indexer_kl_loss(const float* scores, int64_t ld_s, const float* target, int64_t ld_t, int S,
+                        int K, float eps, float* row_loss, float* grad, void* stream);
+
+/*
  * Head-averaged attention distribution over the selected slots:
  *   target[i,t] = (1/H) sum_h softmax_t(p_out[i,h,:] * sm_scale)[t]
  * Replaces triton_attn_dist, dsa_fused_kernels.py:1844-1955.  `ld_s` / `ld_h` are the element

@@ -33,6 +33,7 @@ SIGNATURES = {
     "dsa_sparse_mla_bwd_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "dsa_sparse_mla_bwd_workspace_bytes_min": (_sz, [_i, _i, _i, _i]),
     "dsa_sparse_mla_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _vp, _vp, _vp, _sz, _vp]),
+    "dsa_indexer_kl_loss": (_i, [_vp, _i64, _vp, _i64, _i, _i, _f, _vp, _vp, _vp]),
     "dsa_attn_dist": (_i, [_vp, _i, _i, _i, _i, _i64, _i64, _f, _vp, _vp]),
     "dsa_attn_dist_qk": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp, _vp]),
     "dsa_mla_absorb": (_i, [_vp, _i64, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _i, _vp]),

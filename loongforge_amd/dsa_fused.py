@@ -568,8 +568,9 @@ class DSAttentionFused(MegatronModule):
         if need_loss:
             indexer_loss_coeff = getattr(self.config, "dsa_indexer_loss_coeff", 0.0)
             main_attn_probs = main_attn_probs[:, : index_scores.shape[-1]]
-            index_attn_probs = torch.softmax(index_scores, dim=-1)
-            loss = F.kl_div((index_attn_probs + 1e-10).log(), main_attn_probs.float() + 1e-10, reduction="sum")
+            # softmax, F.kl_div(log(pred + 1e-10), target + 1e-10, "sum") and their backward in one kernel
+            from . import ops
+            loss = ops.indexer_kl_loss(index_scores, main_attn_probs, 1e-10)
             indexer_loss = indexer_loss_coeff * loss / sq
             if indexer_loss_coeff > 0:
                 DSAIndexerLossLoggingHelperFused.save_loss_to_tracker(

@@ -666,6 +666,55 @@ def attn_dist_qk(q, kv, ids, lse, q_start: int, sm_scale: float, heads_in_mean: 
 ROPE_ADJACENT, ROPE_SPLIT = 0, 1   # where pair i sits in a row: (2i, 2i+1) or (i, i + emb_dim/2)
 
 
+@torch.library.custom_op("dsa::indexer_kl_loss", mutates_args=())
+def _kl_loss_op(scores: torch.Tensor, target: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    _need_gpu(scores, target)
+    if scores.ndim != 2 or target.shape != scores.shape:
+        raise ValueError("indexer_kl_loss expects scores and target of one shape [S, K]")
+    S, K = scores.shape
+    scores = scores.float()
+    target = target.float()
+    if scores.stride(1) != 1:
+        scores = scores.contiguous()
+    if target.stride(1) != 1:
+        target = target.contiguous()
+    row_loss = torch.empty(S, dtype=torch.float32, device=scores.device)
+    grad = torch.empty(S, K, dtype=torch.float32, device=scores.device)
+    lib = _lib.load()
+    with torch.cuda.device(scores.device):
+        _lib.check(lib.dsa_indexer_kl_loss(scores.data_ptr(), scores.stride(0) if S > 1 else K, target.data_ptr(),
+                                           target.stride(0) if S > 1 else K, S, K, float(eps), row_loss.data_ptr(),
+                                           grad.data_ptr(), _stream(scores)), "dsa_indexer_kl_loss")
+    return row_loss, grad
+
+
+@_kl_loss_op.register_fake
+def _(scores, target, eps):
+    return scores.new_empty(scores.shape[0], dtype=torch.float32), scores.new_empty(scores.shape, dtype=torch.float32)
+
+
+class _IndexerKLLoss(torch.autograd.Function):
+    """The loss and its gradient come out of the same kernel; backward only scales what forward kept."""
+
+    @staticmethod
+    def forward(ctx, scores, target, eps):
+        row_loss, grad = _kl_loss_op(scores.detach(), target.detach(), eps)
+        ctx.save_for_backward(grad)
+        ctx.in_dtype = scores.dtype
+        return row_loss.sum()
+
+    @staticmethod
+    def backward(ctx, g):
+        (grad,) = ctx.saved_tensors
+        return (grad * g).to(ctx.in_dtype), None, None
+
+
+def indexer_kl_loss(scores: torch.Tensor, target: torch.Tensor, eps: float = 1e-10) -> torch.Tensor:
+    """``F.kl_div((softmax(scores, -1) + eps).log(), target + eps, reduction="sum")`` as one kernel
+    (dsa_fused.py:931-937 of the reference); differentiable in ``scores``, the target is a constant."""
+    return _IndexerKLLoss.apply(scores, target, float(eps))
+
+
 def _rows_view(t: torch.Tensor, what: str):
     """(data_ptr, token stride, head stride) of a [tokens, heads, width] bf16 view with unit inner stride."""
     if t.dtype != torch.bfloat16 or t.ndim != 3 or (t.shape[-1] > 1 and t.stride(-1) != 1):
